@@ -1,0 +1,178 @@
+/* mlk.h - C ABI of the gfx950 (MI355X) native-layout GeMV / narrow-GeMM / fused-MoE kernels.
+ *
+ * One shared library, plain pointers and sizes, no torch types.  Every entry
+ * point replaces one function that the reference exports to Python through its
+ * pybind module (csrc/ffi.cu:32-143); the reference line each one stands in for
+ * is cited beside it.  All pointers are DEVICE pointers unless said otherwise,
+ * all matrices are dense and contiguous, and every call only enqueues work on
+ * `stream` (a hipStream_t passed as void*; NULL = the default stream): nothing
+ * is allocated, nothing is synchronised, no global state is kept besides the
+ * last error text of the calling thread.
+ *
+ * Naming follows the reference: weights are "A" [N rows = output features,
+ * K reduction], activations are "B" [M tokens, K], outputs are "C" [M, N].
+ * (The reference calls these m, k and n.)
+ *
+ * Return value: 0 on success, a negative MLK_ERR_* otherwise; the text of the
+ * last failure is available from mlk_last_error().
+ */
+#ifndef MLK_H_
+#define MLK_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MLK_OK 0
+#define MLK_ERR_INVALID (-1)   /* argument outside what the kernels support  */
+#define MLK_ERR_LAUNCH (-2)    /* the HIP runtime refused the launch          */
+#define MLK_ERR_WORKSPACE (-3) /* workspace too small                         */
+
+/* element kinds */
+#define MLK_F16 0
+#define MLK_BF16 1
+#define MLK_FP8_E4M3 2 /* soft-FP8 weights: one e4m3 byte per element */
+
+/* output placement of the narrow GeMM */
+#define MLK_C_ROWMAJOR 0 /* C[M, N]                               */
+#define MLK_C_NATIVE 1   /* layout-C [N/32, ceil(M/16), 4, 16, 8] */
+
+/* activation placement of the narrow GeMM */
+#define MLK_B_ROWMAJOR 0 /* B[M, K]                               */
+#define MLK_B_NATIVE 1   /* layout-B [K/32, ceil(M/16), 4, 16, 8] */
+
+int mlk_version(void);
+const char *mlk_last_error(void);
+
+/* ------------------------------------------------------------------ relayout
+ * Pure permutations of 16-byte (16-bit elements) or 8-byte (fp8) granules;
+ * bit-exact, any bit pattern. */
+
+/* [N, K] row-major -> layout-A [N/16, K/8, 16, 8].  elem_size 1 or 2.
+ * Stands in for the offline `A.view(m//16,16,k//8,8).permute(0,2,1,3)` of the
+ * reference's scripts (benchmark_and_test/gemv_benchmark.py:47-48) and the
+ * un-exported device packer csrc/moe_kernels/layout.h:58-99.
+ * `batch` independent matrices are processed back to back. */
+int mlk_pack_layout_a(const void *src, void *dst, int64_t batch, int n, int k, int elem_size, void *stream);
+/* inverse of mlk_pack_layout_a */
+int mlk_unpack_layout_a(const void *src, void *dst, int64_t batch, int n, int k, int elem_size, void *stream);
+
+/* B[M, K] row-major (16-bit) -> layout-B [K/32, M/16, 4, 16, 8].
+ * Replaces `layoutB`, csrc/layout_b.cu:65-99 (ffi.cu:36).  M % 16 == 0, K % 32 == 0. */
+int mlk_layout_b(const void *src, void *dst, int m, int k, void *stream);
+
+/* layout-C [N/32, M/16, 4, 16, 8] (16-bit) -> C[M, N] row-major.
+ * Replaces `reLayoutC`, csrc/re_layout_c.cu:63-95 (ffi.cu:37).  Any M % 16 == 0
+ * (the reference launches an empty grid when M/16 > 104). */
+int mlk_re_layout_c(const void *src, void *dst, int m, int n, void *stream);
+
+/* Swap bytes 1 and 2 of every dword of `nbytes` bytes (nbytes % 4 == 0).
+ * Replaces `fp8_weight_repack`, csrc/fp8_weight_repack.cu:44-67 (ffi.cu:92-93);
+ * covers the whole tensor (the reference skips partial 256x256 blocks). */
+int mlk_fp8_weight_repack(const void *src, void *dst, int64_t nbytes, void *stream);
+
+/* ---------------------------------------------------------------------- GeMV
+ * y[M, N] = T(alpha * x[M, K] . A^T (+ bias[N])), 1 <= M <= 4, fp32 accumulate,
+ * A in layout-A.  Replaces `gemv_layoutA` / `gemv_layoutA_wapper`,
+ * csrc/gemv_layout_a.cu:17-150 (ffi.cu:65-67, :87-91), which only takes M = 1.
+ *
+ * a_kind MLK_F16 / MLK_BF16 (x and y have the same kind) or MLK_FP8_E4M3 with
+ * x_kind MLK_BF16 and `scale` = fp32 [ceil(N/128), ceil(K/128)] (may be NULL = 1).
+ * N % 16 == 0, K % 32 == 0 (K % 64 == 0 for fp8).
+ * Launch parameters (what the reference's csv rows select):
+ *   block_dim_x  threads per workgroup, 64..1024, multiple of 64
+ *   kernel_id    1 = streaming kernel (the only one)
+ *   p1           row groups (of 16 rows) per workgroup, >= 1, divides N/16... see DESIGN
+ *   p2           loads kept in flight per wave, 1..8
+ */
+int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k, int a_kind, int x_kind,
+                      float alpha, const void *bias, const float *scale, int block_dim_x, int kernel_id, int p1,
+                      int p2, void *stream);
+
+/* --------------------------------------------------------------- narrow GeMM
+ * C = T(alpha * B . A^T (+ bias[N])), 1 <= M <= 256, A in layout-A, MFMA
+ * 16x16x32 with fp32 accumulation.
+ *
+ *   b_mode MLK_B_ROWMAJOR, c_mode MLK_C_ROWMAJOR : `gemm_layoutA` / `_wapper`
+ *       csrc/gemm_layout_A.cu:684-787 (ffi.cu:43-45, :74-78) and, with
+ *       a_kind MLK_FP8_E4M3 + scale, `gemm_layoutA_soft_fp8` / `_wapper`
+ *       csrc/gemm_layout_A_soft_fp8.cu:749-862 (ffi.cu:46-48, :79-83)
+ *   b_mode MLK_B_NATIVE,   c_mode MLK_C_ROWMAJOR : `gemm_layoutAB_ContinuousC`
+ *       csrc/gemm_layout_ab_continuous_c.cu:1051-1093 (ffi.cu:49-51, :84-86)
+ *   b_mode MLK_B_NATIVE,   c_mode MLK_C_NATIVE   : `gemm_layoutABC`
+ *       csrc/gemm_layout_abc.cu:754-791 (ffi.cu:38-39, :68-73)
+ *
+ * With a native B or C, M must be a multiple of 16.  N % 16 == 0, K % 32 == 0
+ * (K % 64 == 0 for fp8 weights; N % 32 == 0 for a native C).
+ * Launch parameters: kernel_id 1; p1 = row groups per wave (1, 2 or 4);
+ * p2 = waves per workgroup that split K (1, 2, 4, 8 or 16); p3 = K splits across
+ * workgroups (>= 1; > 1 needs `workspace`).
+ * workspace: device scratch of at least mlk_gemm_workspace_bytes() bytes, only
+ * read and written inside the call (contents need not be preserved, but the
+ * first `mlk_gemm_counter_bytes()` bytes must be zero before the first call and
+ * are left zero by every call).  May be NULL when p3 == 1. */
+int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, int n, int k, int a_kind, int x_kind,
+                      int b_mode, int c_mode, float alpha, const void *bias, const float *scale, int kernel_id,
+                      int p1, int p2, int p3, void *workspace, size_t workspace_bytes, void *stream);
+size_t mlk_gemm_workspace_bytes(int m, int n, int p1, int p3);
+size_t mlk_gemm_counter_bytes(void);
+
+/* ----------------------------------------------------------------------- MoE */
+
+/* Router: scores (score_fun 0 = softmax, 1 = sigmoid), optional correction
+ * bias for selection, grouped selection, top-K with ties to the lower id.
+ * Replaces `fused_routing_gate`, csrc/moe_kernels/fused_gating.cu:5-67 ->
+ * fused_topK.h:21-607 (ffi.cu:102-105).  logits [T, E] of kind x_kind,
+ * ids int32 [T, K], weights x_kind [T, K] (un-biased scores; renormalised in
+ * the weights' own precision when `renormalize` != 0, which the reference
+ * leaves to its Python caller, muxi_moe_planC.py:69-70).
+ * E <= 256, topk <= 32, n_groups divides E, topk_groups <= n_groups. */
+int mlk_fused_routing_gate(const void *logits, int x_kind, int score_fun, int n_tokens, int n_experts,
+                           int n_groups, int topk_groups, int topk, const void *bias, int renormalize,
+                           int32_t *ids, void *weights, void *stream);
+
+/* Token -> expert-block alignment.  Replaces
+ * `batched_routed_activation_indexed_to_expert_block_indexed`,
+ * csrc/moe_kernels/fused_experts_compute.cu:6-48 -> moe_align_tokens.h:8-94,
+ * moe_align_tokens.cu:5-21 (ffi.cu:106-111).
+ *   topk_ids            int32 [n_pairs]           (n_pairs = T * K)
+ *   sorted_token_ids    int32 [n_pairs + E*(block-1)]; every slot is written
+ *                       (routed pairs ascending inside each expert, sentinel
+ *                       n_pairs elsewhere) - no pre-fill needed
+ *   cumsum_buffer       int32 [E + 1]; on return cumsum[e] + count[e] for
+ *                       e < E and the padded total at [E], as the reference's
+ *                       atomic cursors leave it
+ *   padded_num_blocks   int32 [1]
+ *   experts_ids         int32 [ceil((n_pairs + E*(block-1)) / block)]
+ *   experts_map         int32 [E_global] or NULL; -1 drops the pair
+ * block must be 16. */
+int mlk_moe_align_tokens(const int32_t *topk_ids, int n_pairs, int n_experts, int block,
+                         const int32_t *experts_map, int32_t *sorted_token_ids, int32_t *cumsum_buffer,
+                         int32_t *padded_num_blocks, int32_t *experts_ids, void *stream);
+
+/* Expert compute on an aligned batch: grouped gate/up GeMM with SiLU(gate)*up,
+ * grouped down GeMM, routing-weighted sum back into token order.  Replaces both
+ * overloads of `fused_experts_compute`,
+ * csrc/moe_kernels/fused_experts_compute.cu:50-296 (ffi.cu:112-143).
+ *   w1 [E, 2I, H] and w2 [E, H, I], each expert slab in layout-A; w_kind
+ *   MLK_F16 / MLK_BF16 (= x_kind) or MLK_FP8_E4M3 with x_kind MLK_BF16 and fp32
+ *   scales w1_scale [E, 2I/128, H/128], w2_scale [E, H/128, I/128]
+ *   x [T, H], topk_weights [T*K] of x_kind, y [T, H] of x_kind (overwritten)
+ *   sorted_token_ids / padded_num_blocks / experts_ids from mlk_moe_align_tokens
+ *   workspace: at least mlk_moe_workspace_bytes() bytes of device scratch.
+ * H % 128 == 0, I % 128 == 0. */
+int mlk_fused_experts_compute(const void *w1, const void *w2, const void *x, int n_tokens, int n_experts,
+                              int topk, int hidden, int inter, int w_kind, int x_kind,
+                              const void *topk_weights, const int32_t *sorted_token_ids,
+                              const int32_t *padded_num_blocks, const int32_t *experts_ids,
+                              const float *w1_scale, const float *w2_scale, void *y, void *workspace,
+                              size_t workspace_bytes, void *stream);
+size_t mlk_moe_workspace_bytes(int n_tokens, int n_experts, int topk, int hidden, int inter);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MLK_H_ */

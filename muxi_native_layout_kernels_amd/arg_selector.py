@@ -1,0 +1,162 @@
+"""csv-driven launch-parameter dispatch for gfx950.
+
+Host-side mirror of the reference's seven selectors (csrc/arg_selector.cu:14-540,
+csrc/arg_selector.h:9-125).  Same file names, same column layout and the same
+parse rules: the first line is a header, cells are integers separated by ',',
+rows with the wrong number of cells are reported and skipped, a later row with
+the same key replaces an earlier one.  A shape that is not in its table gets a
+one-time warning and a fallback that is remembered for the rest of the process
+(arg_selector.cu:63-72, :207-224).  The tables are immutable after loading; the
+miss memo is kept under a lock.
+
+What the columns select on gfx950 (the rows are produced by the scripts in
+`kernel_args_scan/`):
+
+  GeMV tables   m,k -> BLOCK_DIM_X, KernelId, KernelParam1, KernelParam2
+                BLOCK_DIM_X  threads per workgroup (64..1024)
+                KernelId     1 = streaming GeMV
+                KernelParam1 row groups (16 rows) per workgroup
+                KernelParam2 16-byte loads kept in flight per wave
+  GEMM tables   m,n,k -> kernelId, kernelParam1, kernelParam2, kernelParam3
+                kernelId     1 = wave-tiled MFMA kernel
+                kernelParam1 row groups per wave (1, 2, 4)
+                kernelParam2 waves per workgroup splitting K (1..16)
+                kernelParam3 K splits across workgroups
+"""
+import os
+import sys
+import threading
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+GEMM_FALLBACK = (1, 1, 1, 1)
+GEMV_FALLBACK = (256, 1, 1, 1)
+
+
+class _Selector:
+    def __init__(self, filename, key_cells, fallback, label, heuristic=None):
+        self.filename = filename
+        self.key_cells = key_cells
+        self.fallback = fallback
+        self.label = label
+        self.heuristic = heuristic
+        self._table = None
+        self._memo = {}
+        self._lock = threading.Lock()
+
+    def path(self):
+        return os.path.join(_HERE, self.filename)
+
+    def _load(self):
+        table = {}
+        try:
+            with open(self.path(), "r") as f:
+                lines = f.read().splitlines()
+        except OSError:
+            sys.stderr.write("Error opening file: %s\n" % self.path())
+            sys.stderr.write("All %s shape will fallback to default args\n" % self.label)
+            lines = []
+        for line in lines[1:]:
+            if not line.strip():
+                continue
+            try:
+                cells = [int(c) for c in line.split(",")]
+            except ValueError:
+                sys.stderr.write("Invalid line: %s\n" % line)
+                continue
+            if len(cells) != self.key_cells + 4:
+                sys.stderr.write("Invalid line: %s\n" % line)
+                continue
+            table[tuple(cells[:self.key_cells])] = tuple(cells[self.key_cells:])
+        return table
+
+    def table(self):
+        if self._table is None:
+            with self._lock:
+                if self._table is None:
+                    self._table = self._load()
+        return self._table
+
+    def get_args(self, key):
+        key = tuple(int(v) for v in key)
+        hit = self.table().get(key)
+        if hit is not None:
+            return hit
+        with self._lock:
+            memo = self._memo.get(key)
+            if memo is not None:
+                return memo
+            args = self.heuristic(*key) if self.heuristic is not None else self.fallback
+            sys.stderr.write(" Warning: No matching arguments found for %s shape: %s. Fallback args to %s\n" %
+                             (self.label, ", ".join(str(v) for v in key), ",".join(str(v) for v in args)))
+            self._memo[key] = args
+            return args
+
+
+def _gemv_default(n, k):
+    """Fallback for a GeMV shape that was never scanned: one row group per
+    workgroup, enough waves that the grid holds >= 8 waves per CU, 4 loads in flight."""
+    groups = max(1, n // 16)
+    waves = 4
+    while waves < 16 and groups * waves < 256 * 8:
+        waves *= 2
+    return (waves * 64, 1, 1, 4)
+
+
+def _gemm_default(n, m, k):
+    """Fallback for a GEMM shape that was never scanned."""
+    groups = max(1, n // 16)
+    r = 1 if m > 32 else 2
+    if groups % r:
+        r = 1
+    waves = 1
+    while waves < 16 and (groups // r) * waves < 256 * 8:
+        waves *= 2
+    return (1, r, waves, 1)
+
+
+_SELECTORS = {
+    # reference getters: csrc/arg_selector.cu:84-87 (layout gemm), :158-161 (continuous C),
+    # :236-239 (gemv fp16), :312-315 (layoutA gemm), :389-392 (layoutA soft fp8), :464-467 (soft-fp8 gemv),
+    # :537-540 (bf16 gemv)
+    "layout_gemm": _Selector("layout_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK, "layout GEMM", _gemm_default),
+    "continuous_gemm": _Selector("continuous_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK, "ContinuousC GEMM",
+                                 _gemm_default),
+    "layoutA_gemm": _Selector("layoutA_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK, "layoutA GEMM", _gemm_default),
+    "layoutA_soft_fp8_gemm": _Selector("layoutA_Soft_Fp8_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK,
+                                       "layoutA soft-FP8 GEMM", _gemm_default),
+    "gemv_fp16": _Selector("layout_gemv_dispatch_arg.csv", 2, GEMV_FALLBACK, "GEMV", _gemv_default),
+    "gemv_bf16": _Selector("layout_gemv_bf16_dispatch_arg.csv", 2, GEMV_FALLBACK, "bf16 GEMV", _gemv_default),
+    "gemv_soft_fp8": _Selector("layout_gemv_soft_fp8_dispatch_arg.csv", 2, GEMV_FALLBACK, "soft-FP8 GEMV",
+                               _gemv_default),
+}
+
+
+def selector(name):
+    return _SELECTORS[name]
+
+
+def gemv_guard(args, n, k):
+    """Guard rails applied after the GeMV lookup (csrc/gemv_layout_a.cu:132-143): a row
+    that asks for more row groups per workgroup than divide N/16, or more than
+    the wave count allows, is replaced by the plain configuration."""
+    block, kid, p1, p2 = args
+    if kid != 1 or p1 < 1 or (n // 16) % p1 != 0 or (block // 64) % p1 != 0 or block % 64 or not 64 <= block <= 1024:
+        return (256, 1, 1, 4)
+    return args
+
+
+def parse_table_text(text, key_cells):
+    """Parse csv text with the selector's rules (used by the scan scripts and the tests)."""
+    table = {}
+    for line in text.splitlines()[1:]:
+        if not line.strip():
+            continue
+        try:
+            cells = [int(c) for c in line.split(",")]
+        except ValueError:
+            continue
+        if len(cells) != key_cells + 4:
+            continue
+        table[tuple(cells[:key_cells])] = tuple(cells[key_cells:])
+    return table

@@ -1,0 +1,115 @@
+// Shared device helpers for the gfx950 native-layout kernels.
+//
+// Everything here is written for CDNA4 only: 64-lane wavefronts, 16-byte
+// global loads, v_dot2 / v_mfma 16x16x32 for 16-bit operands and the hardware
+// OCP-fp8 converter for the soft-FP8 weights.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mlk.h"
+
+namespace mlk {
+
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
+typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+constexpr int kWave = 64;
+
+// Record an error message for mlk_last_error() and return the code.
+int fail(int code, const char *msg);
+
+#define MLK_REQUIRE(cond, msg)                                                  \
+    do {                                                                        \
+        if (!(cond)) return ::mlk::fail(MLK_ERR_INVALID, msg);                  \
+    } while (0)
+
+#define MLK_LAUNCH_CHECK()                                                      \
+    do {                                                                        \
+        hipError_t e__ = hipGetLastError();                                     \
+        if (e__ != hipSuccess) return ::mlk::fail(MLK_ERR_LAUNCH, hipGetErrorString(e__)); \
+    } while (0)
+
+// ---------------------------------------------------------------- conversions
+__device__ __forceinline__ float bf16_bits_to_f32(uint32_t b) { return __uint_as_float(b << 16); }
+
+// fp32 -> bf16 bits, round to nearest even (NaN kept quiet).
+__device__ __forceinline__ uint32_t f32_to_bf16_bits(float f) {
+    uint32_t u = __float_as_uint(f);
+    if ((u & 0x7fffffffu) > 0x7f800000u) return (u >> 16) | 0x40u;
+    return (u + 0x7fffu + ((u >> 16) & 1u)) >> 16;
+}
+
+__device__ __forceinline__ uint32_t f32_to_f16_bits(float f) {
+    _Float16 h = (_Float16)f;
+    return (uint32_t)__builtin_bit_cast(unsigned short, h);
+}
+
+__device__ __forceinline__ float f16_bits_to_f32(uint32_t b) {
+    return (float)__builtin_bit_cast(_Float16, (unsigned short)b);
+}
+
+// Element traits for the two 16-bit activation/output types.
+struct F16 {
+    static constexpr int kind = MLK_F16;
+    __device__ static __forceinline__ float to_f32(uint32_t b) { return f16_bits_to_f32(b); }
+    __device__ static __forceinline__ uint32_t from_f32(float f) { return f32_to_f16_bits(f); }
+    // acc += a.lo*b.lo + a.hi*b.hi with fp32 accumulation
+    __device__ static __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2, a), __builtin_bit_cast(f16x2, b), acc, false);
+    }
+    __device__ static __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(f16x8, a), __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
+    }
+};
+
+struct BF16 {
+    static constexpr int kind = MLK_BF16;
+    __device__ static __forceinline__ float to_f32(uint32_t b) { return bf16_bits_to_f32(b); }
+    __device__ static __forceinline__ uint32_t from_f32(float f) { return f32_to_bf16_bits(f); }
+    __device__ static __forceinline__ float dot2(uint32_t a, uint32_t b, float acc) {
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, a), __builtin_bit_cast(bf16x2, b), acc, false);
+    }
+    __device__ static __forceinline__ f32x4 mfma(u32x4 a, u32x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8, a), __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
+    }
+};
+
+// ------------------------------------------------------------- soft-FP8 widening
+// Four e4m3 bytes (one dword, byte 0 = lowest k) -> two dwords of packed bf16
+// pairs {k0,k1} and {k2,k3}: W = trunc_bf16(fp32(e4m3) * scale).  The hardware
+// converter yields the exact fp32 value of each OCP e4m3 byte; one fp32 multiply
+// by the block scale and a byte permute that keeps the upper halves reproduces
+// the reference's "widen, multiply by 2^120*scale, drop the low 16 bits"
+// (csrc/utils.cuh:80-99) for every non-NaN code and |scale| < 2^8.
+__device__ __forceinline__ void fp8x4_to_bf16x4(uint32_t w, float scale, uint32_t &lo, uint32_t &hi) {
+    f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+    f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8((int)w, true);
+    float a0 = a[0] * scale, a1 = a[1] * scale, b0 = b[0] * scale, b1 = b[1] * scale;
+    // v_perm_b32 selector: bytes 3,2 of the second source then bytes 3,2 of the first
+    lo = __builtin_amdgcn_perm(__float_as_uint(a1), __float_as_uint(a0), 0x07060302u);
+    hi = __builtin_amdgcn_perm(__float_as_uint(b1), __float_as_uint(b0), 0x07060302u);
+}
+
+// 64-lane xor shuffle of an fp32 through the LDS crossbar (no LDS memory used).
+__device__ __forceinline__ float lane_xor(float v, int mask) {
+    int lane = __lane_id();
+    return __int_as_float(__builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, __float_as_int(v)));
+}
+
+__device__ __forceinline__ u32x4 ld_global_u32x4(const void *p) { return *reinterpret_cast<const u32x4 *>(p); }
+__device__ __forceinline__ u32x4 ld_stream_u32x4(const void *p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(p));
+}
+__device__ __forceinline__ u32x2 ld_stream_u32x2(const void *p) {
+    return __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(p));
+}
+
+}  // namespace mlk

@@ -1,0 +1,320 @@
+// Narrow GeMM (1 <= M <= 64 per weight pass) over layout-A weights with
+// v_mfma_f32_16x16x32: C[M, N] = alpha * B[M, K] . A^T + bias.
+//
+// Work decomposition.  A workgroup owns R consecutive row groups (16 R weight
+// rows) and one of SK slices of K.  Its WK waves take the slice's 32-wide k
+// tiles round-robin.  For every k tile a wave loads R weight fragments (1 KiB
+// each, 16 bytes per lane, coalesced, non-temporal) and CB activation
+// fragments (CB = ceil(M/16) <= 4) and issues R*CB MFMAs, so each activation
+// fragment is reused R times and each weight fragment CB times; weights are
+// read from HBM exactly once.  Fragments are prefetched U tiles ahead in a
+// register ring.  Wave partials are folded through LDS in wave order; with
+// SK > 1 workgroup partials go to an fp32 workspace and the last workgroup to
+// arrive for a row tile folds them in slice order, so results are
+// deterministic and never depend on atomics in the data path.
+//
+// The same kernel serves the three operand placements of the reference:
+// row-major or layout-B activations, row-major or layout-C output.  Because
+// the accumulation order is identical, layout-C output followed by the
+// layout-C -> row-major permutation equals the row-major output bit for bit.
+//
+// Algorithmic traffic per call: N*K*sizeof(W) (+ scales) + M*K*2 + M*N*2 bytes.
+#include "mlk_gemm_tile.cuh"
+
+namespace mlk {
+
+constexpr size_t kCounterBytes = 64 * 1024;
+
+struct GemmArgs {
+    const uint8_t *A;
+    const uint16_t *B;
+    uint16_t *C;
+    const uint16_t *bias;
+    const float *scale;
+    float *partial;      // [SK][row_tiles][R*CB][64] x 4 floats
+    int *counters;       // [row_tiles], zero between calls
+    int M;               // tokens handled by this launch (columns cb0*16 .. )
+    int M_total;         // tokens in the whole problem (row count of B / C)
+    int cb0;             // first 16-token block of this launch
+    int N, K;
+    int WK, SK;
+    float alpha;
+};
+
+// Most threads a workgroup may have for a given accumulator tile count, so that the
+// register file holds the accumulators plus the prefetch ring without spilling.
+__host__ __device__ constexpr int max_threads_for(int ntile) { return ntile <= 4 ? 1024 : (ntile <= 8 ? 512 : 256); }
+
+template <class T, bool FP8, int CB, int R, int BMODE, int CMODE, int U>
+__global__ void __launch_bounds__(max_threads_for(R *CB)) gemm_wave_kernel(GemmArgs p) {
+    extern __shared__ f32x4 red[];  // [WK][R*CB][64]
+    __shared__ int s_last;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int q = lane >> 4, r16 = lane & 15;
+    const int sk = blockIdx.x % p.SK;
+    const int rt = blockIdx.x / p.SK;
+    const int rg0 = rt * R;
+    const int tiles_total = p.K >> 5;
+    const int tiles_per = (tiles_total + p.SK - 1) / p.SK;
+    const int tbeg = sk * tiles_per;
+    const int tend = min(tiles_total, tbeg + tiles_per);
+    const int mb_total = (p.M_total + 15) >> 4;
+    const int scale_cols = (p.K + 127) >> 7;
+    constexpr int WBYTES = FP8 ? 1 : 2;
+
+    const uint8_t *abase[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) abase[r] = p.A + (size_t)(rg0 + r) * p.K * 16 * WBYTES;
+
+    // activation fragment source for this lane
+    const uint16_t *bptr[CB];
+    bool bok[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        if (BMODE == MLK_B_NATIVE) {
+            bptr[cb] = p.B + ((size_t)(p.cb0 + cb) * 64 + lane) * 8;
+            bok[cb] = true;
+        } else {
+            int tok = (p.cb0 + cb) * 16 + r16;
+            bok[cb] = tok < p.M_total;
+            bptr[cb] = p.B + (size_t)(bok[cb] ? tok : 0) * p.K + q * 8;
+        }
+    }
+    const size_t bstep = (BMODE == MLK_B_NATIVE) ? (size_t)mb_total * 512 : 32;  // elements per k tile
+
+    f32x4 acc[R][CB];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int nt = (tbeg + wave < tend) ? (tend - tbeg - wave + p.WK - 1) / p.WK : 0;
+
+    WeightFrag<FP8> wf[U][R];
+    u32x4 bf[U][CB];
+    float sc[U][R];
+    auto issue = [&](int slot, int kt) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
+            if (FP8) sc[slot][r] = p.scale ? p.scale[((rg0 + r) >> 3) * scale_cols + (kt >> 2)] : 1.f;
+        }
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            if (bok[cb]) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * bstep);
+            else bf[slot][cb] = u32x4{0u, 0u, 0u, 0u};
+        }
+    };
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+        if (u < nt) issue(u, tbeg + wave + u * p.WK);
+
+    for (int i = 0; i < nt; i += U) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (i + u < nt) {
+                u32x4 a[R], b[CB];
+#pragma unroll
+                for (int r = 0; r < R; ++r) a[r] = weight_operand<FP8>(wf[u][r], FP8 ? sc[u][r] : 1.f);
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) b[cb] = bf[u][cb];
+                if (i + u + U < nt) issue(u, tbeg + wave + (i + u + U) * p.WK);
+#pragma unroll
+                for (int r = 0; r < R; ++r)
+#pragma unroll
+                    for (int cb = 0; cb < CB; ++cb) acc[r][cb] = T::mfma(a[r], b[cb], acc[r][cb]);
+            }
+        }
+    }
+
+    constexpr int NTILE = R * CB;
+    const int row_tiles = gridDim.x / p.SK;
+
+    auto epilogue = [&](int j, f32x4 v) {
+        const int r = j / CB, cb = j - r * CB;
+        const int n = (rg0 + r) * 16 + 4 * q;
+        const int tok = (p.cb0 + cb) * 16 + r16;
+        if (tok >= p.M_total) return;
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o[i] = p.alpha * v[i];
+            if (p.bias) o[i] += T::to_f32(p.bias[n + i]);
+        }
+        size_t off;
+        if (CMODE == MLK_C_NATIVE)
+            off = ((((size_t)(n >> 5) * mb_total + (tok >> 4)) * 4 + ((n & 31) >> 3)) * 16 + (tok & 15)) * 8 + (n & 7);
+        else
+            off = (size_t)tok * p.N + n;
+        store4<T>(p.C + off, o[0], o[1], o[2], o[3]);
+    };
+    f32x4 *part = reinterpret_cast<f32x4 *>(p.partial);
+    auto part_at = [&](int s, int j) -> size_t { return (((size_t)s * row_tiles + rt) * NTILE + j) * 64 + lane; };
+
+    if (p.WK == 1) {
+        // a single wave: tiles stay in registers
+        if (p.SK == 1) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) epilogue(r * CB + cb, acc[r][cb]);
+            return;
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) part[part_at(sk, r * CB + cb)] = acc[r][cb];
+    } else {
+        // fold the WK waves through LDS in wave order; wave w then owns tiles j = w, w + WK, ...
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) red[(wave * NTILE + r * CB + cb) * 64 + lane] = acc[r][cb];
+        __syncthreads();
+        for (int j = wave; j < NTILE; j += p.WK) {
+            f32x4 v = red[j * 64 + lane];
+            for (int w = 1; w < p.WK; ++w) v += red[(w * NTILE + j) * 64 + lane];
+            if (p.SK == 1) epilogue(j, v);
+            else part[part_at(sk, j)] = v;
+        }
+        if (p.SK == 1) return;
+    }
+
+    // ---- K split across workgroups: the partial is published, the last workgroup to arrive
+    // for this row tile folds all slices in slice order
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int prev = atomicAdd(&p.counters[rt], 1);
+        s_last = (prev == p.SK - 1);
+        if (s_last) p.counters[rt] = 0;
+    }
+    __syncthreads();
+    if (!s_last) return;
+    __threadfence();
+    for (int j = wave; j < NTILE; j += p.WK) {
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < p.SK; ++s) v += part[part_at(s, j)];
+        epilogue(j, v);
+    }
+}
+
+template <class T, bool FP8, int CB, int R, int BMODE, int CMODE>
+static int launch(const GemmArgs &p, hipStream_t s) {
+    constexpr int U = (R * CB >= 8) ? 2 : ((R * CB >= 4) ? 3 : 4);
+    GemmArgs q = p;
+    while (q.WK * 64 > max_threads_for(R * CB) || (size_t)q.WK * R * CB * 1024 > 64 * 1024) q.WK >>= 1;
+    int row_tiles = (q.N / 16) / R;
+    int grid = row_tiles * q.SK;
+    size_t lds = q.WK > 1 ? (size_t)q.WK * R * CB * 1024 : 0;
+    gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, U><<<grid, q.WK * 64, lds, s>>>(q);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+template <class T, bool FP8, int BMODE, int CMODE>
+static int launch_rc(const GemmArgs &p, int R, int CB, hipStream_t s) {
+#define MLK_CASE(RR, CC) \
+    if (R == RR && CB == CC) return launch<T, FP8, CC, RR, BMODE, CMODE>(p, s);
+    MLK_CASE(1, 1) MLK_CASE(1, 2) MLK_CASE(1, 3) MLK_CASE(1, 4)
+    MLK_CASE(2, 1) MLK_CASE(2, 2) MLK_CASE(2, 3) MLK_CASE(2, 4)
+    MLK_CASE(4, 1) MLK_CASE(4, 2) MLK_CASE(4, 3) MLK_CASE(4, 4)
+#undef MLK_CASE
+    return fail(MLK_ERR_INVALID, "gemm: unsupported (row groups per wave, column blocks)");
+}
+
+template <class T, bool FP8>
+static int launch_modes(const GemmArgs &p, int b_mode, int c_mode, int R, int CB, hipStream_t s) {
+    if (b_mode == MLK_B_ROWMAJOR && c_mode == MLK_C_ROWMAJOR)
+        return launch_rc<T, FP8, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR>(p, R, CB, s);
+    if (!FP8) {
+        if (b_mode == MLK_B_NATIVE && c_mode == MLK_C_ROWMAJOR)
+            return launch_rc<T, false, MLK_B_NATIVE, MLK_C_ROWMAJOR>(p, R, CB, s);
+        if (b_mode == MLK_B_NATIVE && c_mode == MLK_C_NATIVE)
+            return launch_rc<T, false, MLK_B_NATIVE, MLK_C_NATIVE>(p, R, CB, s);
+    }
+    return fail(MLK_ERR_INVALID, "gemm: unsupported operand placement");
+}
+
+}  // namespace mlk
+
+using namespace mlk;
+
+extern "C" size_t mlk_gemm_counter_bytes(void) { return kCounterBytes; }
+
+extern "C" size_t mlk_gemm_workspace_bytes(int m, int n, int p1, int p3) {
+    (void)p1;
+    int cb = (m + 15) / 16;
+    if (cb > 4) cb = 4;
+    if (p3 <= 1) return 0;
+    return kCounterBytes + (size_t)p3 * (size_t)(n / 16) * cb * 1024;
+}
+
+extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, int n, int k, int a_kind, int x_kind,
+                                 int b_mode, int c_mode, float alpha, const void *bias, const float *scale,
+                                 int kernel_id, int p1, int p2, int p3, void *workspace, size_t workspace_bytes,
+                                 void *stream) {
+    MLK_REQUIRE(m >= 0 && n >= 0 && k >= 0, "gemm: negative size");
+    MLK_REQUIRE(n % 16 == 0, "gemm: N % 16 must be 0");
+    MLK_REQUIRE(k % 32 == 0, "gemm: K % 32 must be 0");
+    MLK_REQUIRE(kernel_id == 1, "gemm: unknown kernel id");
+    MLK_REQUIRE(p1 == 1 || p1 == 2 || p1 == 4, "gemm: row groups per wave (p1) must be 1, 2 or 4");
+    MLK_REQUIRE((n / 16) % p1 == 0, "gemm: row groups per wave (p1) must divide N/16");
+    MLK_REQUIRE(p2 == 1 || p2 == 2 || p2 == 4 || p2 == 8 || p2 == 16, "gemm: waves per workgroup (p2) must be 1, 2, 4, 8 or 16");
+    MLK_REQUIRE(p3 >= 1 && p3 <= 64, "gemm: K splits across workgroups (p3) must be 1..64");
+    MLK_REQUIRE(x_kind == MLK_F16 || x_kind == MLK_BF16, "gemm: activations must be fp16 or bf16");
+    MLK_REQUIRE(b_mode == MLK_B_ROWMAJOR || b_mode == MLK_B_NATIVE, "gemm: bad activation placement");
+    MLK_REQUIRE(c_mode == MLK_C_ROWMAJOR || c_mode == MLK_C_NATIVE, "gemm: bad output placement");
+    if (b_mode == MLK_B_NATIVE || c_mode == MLK_C_NATIVE) MLK_REQUIRE(m % 16 == 0, "gemm: native B / C need M % 16 == 0");
+    if (c_mode == MLK_C_NATIVE) MLK_REQUIRE(n % 32 == 0, "gemm: native C needs N % 32 == 0");
+    const bool fp8 = a_kind == MLK_FP8_E4M3;
+    if (fp8) {
+        MLK_REQUIRE(x_kind == MLK_BF16, "gemm: soft-FP8 weights need bf16 activations");
+    } else {
+        MLK_REQUIRE(a_kind == x_kind, "gemm: weights and activations must have the same 16-bit type");
+        MLK_REQUIRE(scale == nullptr, "gemm: a scale matrix is only meaningful for soft-FP8 weights");
+    }
+    if (m == 0 || n == 0) return MLK_OK;
+    MLK_REQUIRE(a && b && c, "gemm: null pointer");
+    int sk = p3;
+    if (sk > k / 32) sk = k / 32 > 0 ? k / 32 : 1;
+    const int cb_max = (m + 15) / 16 < 4 ? (m + 15) / 16 : 4;
+    if (sk > 1) {
+        MLK_REQUIRE(workspace != nullptr, "gemm: a K split across workgroups needs a workspace");
+        MLK_REQUIRE((size_t)(n / 16 / p1) * sizeof(int) <= kCounterBytes, "gemm: too many row tiles for the counter region");
+        size_t need = kCounterBytes + (size_t)sk * (size_t)(n / 16) * cb_max * 1024;
+        if (workspace_bytes < need) return fail(MLK_ERR_WORKSPACE, "gemm: workspace too small");
+    }
+    int wk = p2;  // clamped per launch to what registers and LDS allow
+
+    GemmArgs g;
+    g.A = (const uint8_t *)a;
+    g.B = (const uint16_t *)b;
+    g.C = (uint16_t *)c;
+    g.bias = (const uint16_t *)bias;
+    g.scale = scale;
+    g.counters = (int *)workspace;
+    g.partial = workspace ? (float *)((uint8_t *)workspace + kCounterBytes) : nullptr;
+    g.M_total = m;
+    g.N = n;
+    g.K = k;
+    g.WK = wk;
+    g.SK = sk;
+    g.alpha = alpha;
+    hipStream_t s = (hipStream_t)stream;
+    // weight passes of at most 64 tokens
+    for (int c0 = 0; c0 < m; c0 += 64) {
+        int mm = m - c0 < 64 ? m - c0 : 64;
+        g.M = mm;
+        g.cb0 = c0 / 16;
+        int cb = (mm + 15) / 16;
+        int rc;
+        if (fp8) rc = launch_modes<BF16, true>(g, b_mode, c_mode, p1, cb, s);
+        else if (x_kind == MLK_F16) rc = launch_modes<F16, false>(g, b_mode, c_mode, p1, cb, s);
+        else rc = launch_modes<BF16, false>(g, b_mode, c_mode, p1, cb, s);
+        if (rc != MLK_OK) return rc;
+    }
+    return MLK_OK;
+}

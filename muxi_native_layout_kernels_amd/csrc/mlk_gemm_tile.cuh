@@ -1,0 +1,57 @@
+// Wave-level building blocks of the narrow GeMM: operand fragments for
+// v_mfma_f32_16x16x32_{f16,bf16} straight from the native layouts.
+//
+// Fragment maps (lane = 16 q + r):
+//   weights     lane holds row r, k = 32 t + 8 q .. +7  -> 16 bytes at tile + 16*lane of layout-A
+//               (8 bytes at tile + 8*lane for fp8, widened in registers)
+//   activations lane holds token r, same k              -> 16 bytes at tile + 16*lane of layout-B,
+//               or 16 bytes of row r of a row-major [M, K] matrix
+//   accumulator lane holds token r, weight rows 4 q .. 4 q + 3
+#pragma once
+
+#include "mlk_common.cuh"
+
+namespace mlk {
+
+// One k-tile (32 k) of weights for one row group, as an MFMA operand.
+template <bool FP8>
+struct WeightFrag {
+    u32x4 v;
+};
+template <>
+struct WeightFrag<true> {
+    u32x2 v;
+};
+
+template <bool FP8>
+__device__ __forceinline__ WeightFrag<FP8> load_weight_frag(const uint8_t *rg_base, int kt, int lane) {
+    WeightFrag<FP8> f;
+    if constexpr (FP8) f.v = ld_stream_u32x2(rg_base + (size_t)kt * 512 + lane * 8);
+    else f.v = ld_stream_u32x4(rg_base + (size_t)kt * 1024 + lane * 16);
+    return f;
+}
+
+template <bool FP8>
+__device__ __forceinline__ u32x4 weight_operand(const WeightFrag<FP8> &f, float scale) {
+    if constexpr (FP8) {
+        u32x4 o;
+        uint32_t a, b, c, d;
+        fp8x4_to_bf16x4(f.v[0], scale, a, b);
+        fp8x4_to_bf16x4(f.v[1], scale, c, d);
+        o[0] = a; o[1] = b; o[2] = c; o[3] = d;
+        return o;
+    } else {
+        return f.v;
+    }
+}
+
+// Store 4 consecutive outputs (weight rows n .. n+3 of one token) as 8 bytes.
+template <class T>
+__device__ __forceinline__ void store4(uint16_t *p, float a, float b, float c, float d) {
+    u32x2 o;
+    o[0] = T::from_f32(a) | (T::from_f32(b) << 16);
+    o[1] = T::from_f32(c) | (T::from_f32(d) << 16);
+    *reinterpret_cast<u32x2 *>(p) = o;
+}
+
+}  // namespace mlk

@@ -1,0 +1,233 @@
+// Weight-stationary GeMV over layout-A weights: a pure HBM-streaming kernel.
+//
+// A row group (16 weight rows) is one contiguous run of K*32 bytes (K*16 for
+// fp8).  A workgroup owns `G` consecutive row groups; `WK` waves share one row
+// group and take its 1 KiB tiles round-robin, so the workgroup always reads a
+// contiguous window of G*WK KiB.  Every lane issues 16-byte loads at
+// `tile + lane*16` (fully coalesced, non-temporal), keeps `U` of them in flight
+// in a register ring, and multiplies by the matching 8 activations read from
+// LDS (the activation vector is staged there once per workgroup).  Products
+// are accumulated in fp32 with v_dot2; no matrix-core instruction is used.
+// Lane partials are folded with cross-lane shuffles, wave partials through
+// LDS in a fixed order, so the result is deterministic and needs neither
+// atomics nor a zero-filled output.
+//
+// Algorithmic traffic per call: N*K*sizeof(W) weight bytes (+ 4 bytes per
+// 128x128 block of scales) + M*K*2 + M*N*2.
+#include "mlk_common.cuh"
+
+namespace mlk {
+
+constexpr int kXsBytes = 48 * 1024;  // LDS window for the staged activations
+
+template <class T, bool FP8, int M, int U>
+__global__ void __launch_bounds__(1024)
+    gemv_stream_kernel(const uint8_t *__restrict__ A, const uint16_t *__restrict__ X, uint16_t *__restrict__ Y,
+                       int n_groups, int K, int KC, float alpha, const uint16_t *__restrict__ bias,
+                       const float *__restrict__ scale, int G, int WK) {
+    extern __shared__ u32x4 xs[];                 // [M][KC/8] granules of 8 activations
+    __shared__ float red[16 * 16 * M];            // [wave][row][m]
+
+    constexpr int TK = FP8 ? 64 : 32;             // k covered by one 1 KiB tile
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int rg_local = wave / WK;
+    const int ks = wave - rg_local * WK;
+    const int rg = blockIdx.x * G + rg_local;
+    const bool active = rg < n_groups;
+    const int N = n_groups * 16;
+    const int tiles_total = K / TK;
+    const int scale_cols = (K + 127) >> 7;
+
+    // lane -> (k octet inside the tile) ; for 16-bit weights the lane holds row lane&15,
+    // for fp8 it holds the row pair 2*(lane&7), 2*(lane&7)+1.
+    const int oct = FP8 ? (lane >> 3) : (lane >> 4);
+
+    float acc[FP8 ? 2 : 1][M];
+#pragma unroll
+    for (int a = 0; a < (FP8 ? 2 : 1); ++a)
+#pragma unroll
+        for (int m = 0; m < M; ++m) acc[a][m] = 0.f;
+
+    const u32x4 *arow = reinterpret_cast<const u32x4 *>(A) + (size_t)(active ? rg : 0) * tiles_total * 64 + lane;
+    const int stride = WK * 64;                   // u32x4 units between this wave's tiles
+
+    for (int kc0 = 0; kc0 < K; kc0 += KC) {
+        const int kc_len = min(KC, K - kc0);
+        const int t0 = kc0 / TK;
+        const int tiles_here = kc_len / TK;
+        const int nt = (active && ks < tiles_here) ? (tiles_here - ks + WK - 1) / WK : 0;
+        const u32x4 *ap = arow + (size_t)(t0 + ks) * 64;
+
+        // start the weight stream before touching the activations
+        u32x4 buf[U];
+        float sc[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            if (u < nt) {
+                buf[u] = ld_stream_u32x4(ap + (size_t)u * stride);
+                if (FP8) sc[u] = scale ? scale[(rg >> 3) * scale_cols + ((t0 + ks + u * WK) >> 1)] : 1.f;
+            }
+        }
+
+        if (kc0 > 0) __syncthreads();             // everyone is done with the previous window
+        const int granules = kc_len >> 3;
+        for (int i = threadIdx.x; i < M * granules; i += blockDim.x) {
+            int m = i / granules, g = i - m * granules;
+            xs[m * (KC >> 3) + g] = *reinterpret_cast<const u32x4 *>(X + (size_t)m * K + kc0 + g * 8);
+        }
+        __syncthreads();
+
+        for (int i = 0; i < nt; i += U) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (i + u < nt) {
+                    u32x4 cur = buf[u];
+                    float s = FP8 ? sc[u] : 1.f;
+                    const int kt = ks + (i + u) * WK;             // tile index inside the window
+                    if (i + u + U < nt) {
+                        buf[u] = ld_stream_u32x4(ap + (size_t)(i + u + U) * stride);
+                        if (FP8) sc[u] = scale ? scale[(rg >> 3) * scale_cols + ((t0 + kt + U * WK) >> 1)] : 1.f;
+                    }
+                    const int xg = kt * (TK / 8) + oct;            // granule of 8 activations
+                    if (FP8) {
+                        uint32_t w0[4], w1[4];
+                        fp8x4_to_bf16x4(cur[0], s, w0[0], w0[1]);
+                        fp8x4_to_bf16x4(cur[1], s, w0[2], w0[3]);
+                        fp8x4_to_bf16x4(cur[2], s, w1[0], w1[1]);
+                        fp8x4_to_bf16x4(cur[3], s, w1[2], w1[3]);
+#pragma unroll
+                        for (int m = 0; m < M; ++m) {
+                            u32x4 xv = xs[m * (KC >> 3) + xg];
+#pragma unroll
+                            for (int d = 0; d < 4; ++d) {
+                                acc[0][m] = T::dot2(w0[d], xv[d], acc[0][m]);
+                                acc[FP8 ? 1 : 0][m] = T::dot2(w1[d], xv[d], acc[FP8 ? 1 : 0][m]);
+                            }
+                        }
+                    } else {
+#pragma unroll
+                        for (int m = 0; m < M; ++m) {
+                            u32x4 xv = xs[m * (KC >> 3) + xg];
+#pragma unroll
+                            for (int d = 0; d < 4; ++d) acc[0][m] = T::dot2(cur[d], xv[d], acc[0][m]);
+                        }
+                    }
+                }
+            }
+        }
+    }
+
+    // fold the k octets held by different lanes of the wave
+#pragma unroll
+    for (int a = 0; a < (FP8 ? 2 : 1); ++a)
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            float v = acc[a][m];
+            if (FP8) v += lane_xor(v, 8);
+            v += lane_xor(v, 16);
+            v += lane_xor(v, 32);
+            acc[a][m] = v;
+        }
+    if (FP8) {
+        if (lane < 8) {
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                red[(wave * 16 + 2 * lane) * M + m] = acc[0][m];
+                red[(wave * 16 + 2 * lane + 1) * M + m] = acc[FP8 ? 1 : 0][m];
+            }
+        }
+    } else {
+        if (lane < 16) {
+#pragma unroll
+            for (int m = 0; m < M; ++m) red[(wave * 16 + lane) * M + m] = acc[0][m];
+        }
+    }
+    __syncthreads();
+
+    // fold the WK waves of each row group in a fixed order, then the epilogue
+    for (int i = threadIdx.x; i < G * 16 * M; i += blockDim.x) {
+        int m = i % M;
+        int row = (i / M) & 15;
+        int gl = i / (16 * M);
+        int g = blockIdx.x * G + gl;
+        if (g < n_groups) {
+            float sum = 0.f;
+            for (int w = 0; w < WK; ++w) sum += red[((gl * WK + w) * 16 + row) * M + m];
+            int col = g * 16 + row;
+            float out = alpha * sum;
+            if (bias) out += T::to_f32(bias[col]);
+            Y[(size_t)m * N + col] = (uint16_t)T::from_f32(out);
+        }
+    }
+}
+
+template <class T, bool FP8, int M>
+static int launch_u(const void *a, const void *x, void *y, int n, int k, float alpha, const void *bias,
+                    const float *scale, int block, int G, int U, hipStream_t s) {
+    const int W = block / 64;
+    const int WK = W / G;
+    const int n_groups = n / 16;
+    const int grid = (n_groups + G - 1) / G;
+    constexpr int TK = FP8 ? 64 : 32;
+    int KC = k;
+    if ((size_t)M * k * 2 > (size_t)kXsBytes) KC = (kXsBytes / (2 * M)) / TK * TK;
+    size_t lds = (size_t)M * KC * 2;
+#define MLK_GEMV_LAUNCH(UU)                                                                                   \
+    gemv_stream_kernel<T, FP8, M, UU><<<grid, block, lds, s>>>((const uint8_t *)a, (const uint16_t *)x,        \
+                                                                  (uint16_t *)y, n_groups, k, KC, alpha,       \
+                                                                  (const uint16_t *)bias, scale, G, WK)
+    switch (U) {
+        case 1: MLK_GEMV_LAUNCH(1); break;
+        case 2: MLK_GEMV_LAUNCH(2); break;
+        case 4: MLK_GEMV_LAUNCH(4); break;
+        case 6: MLK_GEMV_LAUNCH(6); break;
+        case 8: MLK_GEMV_LAUNCH(8); break;
+        default: return fail(MLK_ERR_INVALID, "gemv: loads in flight (p2) must be 1, 2, 4, 6 or 8");
+    }
+#undef MLK_GEMV_LAUNCH
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+template <class T, bool FP8>
+static int launch_m(int m, const void *a, const void *x, void *y, int n, int k, float alpha, const void *bias,
+                    const float *scale, int block, int G, int U, hipStream_t s) {
+    switch (m) {
+        case 1: return launch_u<T, FP8, 1>(a, x, y, n, k, alpha, bias, scale, block, G, U, s);
+        case 2: return launch_u<T, FP8, 2>(a, x, y, n, k, alpha, bias, scale, block, G, U, s);
+        case 3: return launch_u<T, FP8, 3>(a, x, y, n, k, alpha, bias, scale, block, G, U, s);
+        case 4: return launch_u<T, FP8, 4>(a, x, y, n, k, alpha, bias, scale, block, G, U, s);
+        default: return fail(MLK_ERR_INVALID, "gemv: M must be 1..4");
+    }
+}
+
+}  // namespace mlk
+
+using namespace mlk;
+
+extern "C" int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k, int a_kind, int x_kind,
+                                 float alpha, const void *bias, const float *scale, int block_dim_x, int kernel_id,
+                                 int p1, int p2, void *stream) {
+    MLK_REQUIRE(m >= 1 && m <= 4, "gemv: M must be 1..4");
+    MLK_REQUIRE(n >= 0 && k >= 0, "gemv: negative size");
+    MLK_REQUIRE(n % 16 == 0, "GEMV m % 16(at least) must be 0");
+    MLK_REQUIRE(k % 32 == 0, "GEMV k % 32(at least) must be 0");
+    MLK_REQUIRE(kernel_id == 1, "gemv: unknown kernel id");
+    MLK_REQUIRE(block_dim_x >= 64 && block_dim_x <= 1024 && block_dim_x % 64 == 0,
+                "gemv: BLOCK_DIM_X must be a multiple of 64 in 64..1024");
+    MLK_REQUIRE(p1 >= 1 && (block_dim_x / 64) % p1 == 0, "gemv: row groups per workgroup (p1) must divide the wave count");
+    MLK_REQUIRE(x_kind == MLK_F16 || x_kind == MLK_BF16, "gemv: activations must be fp16 or bf16");
+    if (n == 0) return MLK_OK;
+    MLK_REQUIRE(a && x && y, "gemv: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if (a_kind == MLK_FP8_E4M3) {
+        MLK_REQUIRE(x_kind == MLK_BF16, "gemv: soft-FP8 weights need bf16 activations");
+        MLK_REQUIRE(k % 64 == 0, "gemv: soft-FP8 needs K % 64 == 0");
+        return launch_m<BF16, true>(m, a, x, y, n, k, alpha, bias, scale, block_dim_x, p1, p2, s);
+    }
+    MLK_REQUIRE(a_kind == x_kind, "gemv: weights and activations must have the same 16-bit type");
+    MLK_REQUIRE(scale == nullptr, "gemv: a scale matrix is only meaningful for soft-FP8 weights");
+    if (x_kind == MLK_F16) return launch_m<F16, false>(m, a, x, y, n, k, alpha, bias, scale, block_dim_x, p1, p2, s);
+    return launch_m<BF16, false>(m, a, x, y, n, k, alpha, bias, scale, block_dim_x, p1, p2, s);
+}

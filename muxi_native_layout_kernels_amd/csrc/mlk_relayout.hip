@@ -1,0 +1,155 @@
+// Relayout kernels: layout-A pack / unpack, layout-B pack, layout-C unpack and
+// the fp8 byte repack.  All are pure permutations, one 16-byte (or 8-byte)
+// granule per thread, writes coalesced; HBM-bound copies.
+#include "mlk_common.cuh"
+
+namespace mlk {
+
+// --------------------------------------------------------------- error text
+static thread_local char g_err[256] = "";
+
+int fail(int code, const char *msg) {
+    int i = 0;
+    for (; msg[i] && i < 255; ++i) g_err[i] = msg[i];
+    g_err[i] = 0;
+    return code;
+}
+
+// One granule of 8 elements: G = uint4 for 16-bit elements, uint2 for bytes.
+//
+// layout-A: dst granule ((g * K/8 + o) * 16 + r)  <-  src granule (16 g + r) * K/8 + o
+template <typename G, bool PACK>
+__global__ void __launch_bounds__(256) layout_a_kernel(const G *__restrict__ src, G *__restrict__ dst, int64_t total,
+                                                       int n, int octets) {
+    int64_t per_mat = (int64_t)n * octets;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        int64_t mat = i / per_mat;
+        int64_t j = i - mat * per_mat;          // index in native order
+        int r = (int)(j & 15);
+        int64_t go = j >> 4;
+        int o = (int)(go % octets);
+        int64_t g = go / octets;
+        int64_t rm = (g * 16 + r) * octets + o;  // index in row-major order
+        if (PACK) dst[i] = src[mat * per_mat + rm];
+        else dst[mat * per_mat + rm] = src[i];
+    }
+}
+
+// layout-B / layout-C: native granule ((c * M/16 + g) * 64 + 16 q + r) <-> row-major
+// granule (16 g + r) * K/8 + 4 c + q.  PACK: row-major -> native (layoutB);
+// !PACK: native -> row-major (reLayoutC).  The thread index always runs over
+// the destination so stores are coalesced.
+template <bool PACK>
+__global__ void __launch_bounds__(256) layout_b_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst,
+                                                       int64_t total, int mgroups, int octets) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        if (PACK) {
+            int r = (int)(i & 15);
+            int q = (int)((i >> 4) & 3);
+            int64_t cg = i >> 6;
+            int g = (int)(cg % mgroups);
+            int64_t c = cg / mgroups;
+            dst[i] = src[((int64_t)g * 16 + r) * octets + c * 4 + q];
+        } else {
+            int64_t row = i / octets;
+            int oct = (int)(i - row * octets);
+            int g = (int)(row >> 4), r = (int)(row & 15);
+            int c = oct >> 2, q = oct & 3;
+            dst[i] = src[(((int64_t)c * mgroups + g) << 6) + q * 16 + r];
+        }
+    }
+}
+
+__global__ void __launch_bounds__(256) fp8_repack_kernel(const uint32_t *__restrict__ src, uint32_t *__restrict__ dst,
+                                                         int64_t ndwords) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < ndwords;
+         i += (int64_t)gridDim.x * blockDim.x) {
+        uint32_t w = src[i];
+        // bytes [b0, b1, b2, b3] -> [b0, b2, b1, b3]
+        dst[i] = __builtin_amdgcn_perm(w, w, 0x03010200u);
+    }
+}
+
+static inline int grid_for(int64_t total) {
+    int64_t blocks = (total + 255) / 256;
+    const int64_t cap = 256 * 32;  // 32 workgroups per CU is plenty for a copy
+    return (int)(blocks < 1 ? 1 : (blocks > cap ? cap : blocks));
+}
+
+}  // namespace mlk
+
+using namespace mlk;
+
+extern "C" {
+
+int mlk_version(void) { return 1; }
+const char *mlk_last_error(void) { return g_err; }
+
+static int layout_a_common(const void *src, void *dst, int64_t batch, int n, int k, int elem_size, void *stream,
+                           bool pack) {
+    MLK_REQUIRE(batch >= 0 && n >= 0 && k >= 0, "layout-A: negative size");
+    MLK_REQUIRE(n % 16 == 0 && k % 8 == 0, "layout-A: N % 16 and K % 8 must be 0");
+    MLK_REQUIRE(elem_size == 1 || elem_size == 2, "layout-A: element size must be 1 or 2");
+    int64_t total = batch * (int64_t)n * (k / 8);
+    if (total == 0) return MLK_OK;
+    MLK_REQUIRE(src && dst, "layout-A: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    int grid = grid_for(total);
+    if (elem_size == 2) {
+        if (pack) layout_a_kernel<uint4, true><<<grid, 256, 0, s>>>((const uint4 *)src, (uint4 *)dst, total, n, k / 8);
+        else layout_a_kernel<uint4, false><<<grid, 256, 0, s>>>((const uint4 *)src, (uint4 *)dst, total, n, k / 8);
+    } else {
+        if (pack) layout_a_kernel<uint2, true><<<grid, 256, 0, s>>>((const uint2 *)src, (uint2 *)dst, total, n, k / 8);
+        else layout_a_kernel<uint2, false><<<grid, 256, 0, s>>>((const uint2 *)src, (uint2 *)dst, total, n, k / 8);
+    }
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+int mlk_pack_layout_a(const void *src, void *dst, int64_t batch, int n, int k, int elem_size, void *stream) {
+    return layout_a_common(src, dst, batch, n, k, elem_size, stream, true);
+}
+
+int mlk_unpack_layout_a(const void *src, void *dst, int64_t batch, int n, int k, int elem_size, void *stream) {
+    return layout_a_common(src, dst, batch, n, k, elem_size, stream, false);
+}
+
+int mlk_layout_b(const void *src, void *dst, int m, int k, void *stream) {
+    MLK_REQUIRE(m >= 0 && k >= 0, "layoutB: negative size");
+    MLK_REQUIRE(m % 16 == 0, "n must be a multiple of 16");
+    MLK_REQUIRE(k % 32 == 0, "k must be a multiple of 32");
+    int64_t total = (int64_t)m * (k / 8);
+    if (total == 0) return MLK_OK;
+    MLK_REQUIRE(src && dst, "layoutB: null pointer");
+    layout_b_kernel<true><<<grid_for(total), 256, 0, (hipStream_t)stream>>>((const uint4 *)src, (uint4 *)dst, total,
+                                                                           m / 16, k / 8);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+int mlk_re_layout_c(const void *src, void *dst, int m, int n, void *stream) {
+    MLK_REQUIRE(m >= 0 && n >= 0, "reLayoutC: negative size");
+    MLK_REQUIRE(m % 16 == 0, "n must be a multiple of 16");
+    MLK_REQUIRE(n % 32 == 0, "m must be a multiple of 32");
+    int64_t total = (int64_t)m * (n / 8);
+    if (total == 0) return MLK_OK;
+    MLK_REQUIRE(src && dst, "reLayoutC: null pointer");
+    layout_b_kernel<false><<<grid_for(total), 256, 0, (hipStream_t)stream>>>((const uint4 *)src, (uint4 *)dst, total,
+                                                                            m / 16, n / 8);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+int mlk_fp8_weight_repack(const void *src, void *dst, int64_t nbytes, void *stream) {
+    MLK_REQUIRE(nbytes >= 0 && nbytes % 4 == 0, "fp8_weight_repack: byte count must be a multiple of 4");
+    if (nbytes == 0) return MLK_OK;
+    MLK_REQUIRE(src && dst, "fp8_weight_repack: null pointer");
+    int64_t nd = nbytes / 4;
+    fp8_repack_kernel<<<grid_for(nd), 256, 0, (hipStream_t)stream>>>((const uint32_t *)src, (uint32_t *)dst, nd);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,144 @@
+"""GPU parity: narrow GeMM (layoutA / layoutAB_ContinuousC / layoutABC, soft-FP8) against the
+oracle's float64 product on the un-packed weights, rtol = atol = 1e-2, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as ogemm, layouts
+from helpers import randn, pack_a, pack_b, fp8_codes, assert_close, bits
+
+pytestmark = pytest.mark.gpu
+
+RTOL = ATOL = 1e-2
+
+
+@pytest.mark.parametrize("m", [1, 8, 16, 32, 64])
+def test_gemm_layout_a_fp16_config(mlk, m):
+    n, k = 11008, 4096
+    w = randn((n, k), torch.float16, 0.02, 2025)
+    b = randn((m, k), torch.float16, 1.0, 2026 + m)
+    c = mlk.gemm_layoutA(pack_a(w).cuda(), b.cuda())
+    assert c.shape == (m, n) and c.dtype == torch.float16
+    assert_close(c, ogemm.linear_expected(w, b), RTOL, ATOL, "gemm_layoutA M=%d" % m)
+
+
+@pytest.mark.parametrize("m", [1, 3, 15, 17, 33, 48, 63, 65, 100, 130])
+def test_gemm_layout_a_ragged_tokens(mlk, m):
+    n, k = 256, 512
+    w = randn((n, k), torch.bfloat16, 0.05, 1)
+    b = randn((m, k), torch.bfloat16, 1.0, 2)
+    c = mlk.gemm_layoutA(pack_a(w).cuda(), b.cuda())
+    assert_close(c, ogemm.linear_expected(w, b), RTOL, ATOL, "ragged M=%d" % m)
+
+
+@pytest.mark.parametrize("p1,p2,p3", [(1, 1, 1), (1, 4, 1), (2, 2, 1), (4, 4, 1), (1, 16, 1), (2, 8, 1), (1, 1, 4),
+                                      (2, 4, 3), (4, 2, 8), (1, 2, 64)])
+@pytest.mark.parametrize("m", [16, 40, 64])
+def test_gemm_launch_parameters(mlk, p1, p2, p3, m):
+    n, k = 512, 2048
+    w = randn((n, k), torch.bfloat16, 0.02, 3)
+    b = randn((m, k), torch.bfloat16, 1.0, 4)
+    bias = randn((1, n), torch.bfloat16, 1.0, 5)
+    a = pack_a(w).cuda()
+    want = ogemm.linear_expected(w, b, 0.75, bias)
+    c = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.75, kernelParam1=p1, kernelParam2=p2, kernelParam3=p3,
+                                kernelId=1, bias=bias.cuda())
+    assert_close(c, want, RTOL, ATOL, "params")
+    c2 = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.75, kernelParam1=p1, kernelParam2=p2,
+                                 kernelParam3=p3, kernelId=1, bias=bias.cuda())
+    assert torch.equal(c, c2), "K split across workgroups must be deterministic and leave its counters clean"
+
+
+def test_gemm_special_cases(mlk):
+    n = k = 256
+    eye = torch.eye(n, dtype=torch.float16)
+    b = randn((32, k), torch.float16, 1.0, 6)
+    assert torch.equal(mlk.gemm_layoutA(pack_a(eye).cuda(), b.cuda()).cpu(), b)
+    bias = randn((1, n), torch.float16, 1.0, 7)
+    c0 = mlk.gemm_layoutA(pack_a(eye).cuda(), b.cuda(), alpha=0.0, bias=bias.cuda())
+    assert torch.equal(c0.cpu(), bias.expand(32, n))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_native_chain_bit_exact(mlk, dtype):
+    """layoutB -> gemm_layoutABC -> reLayoutC equals gemm_layoutAB_ContinuousC bit for bit (same launch
+    parameters, hence same accumulation order), and both match the oracle."""
+    n, k, m = 1024, 2048, 32
+    w = randn((n, k), dtype, 0.02, 8)
+    b = randn((m, k), dtype, 1.0, 9)
+    a = pack_a(w).cuda()
+    b_nat = mlk.layoutB(b.cuda())
+    assert np.array_equal(bits(b_nat.cpu()), layouts.pack_layout_b(bits(b)))
+    for (p1, p2, p3) in [(1, 4, 1), (2, 2, 2)]:
+        c_nat = mlk.gemm_layoutABC_wapper(a, b_nat, n, m, k, kernelParam1=p1, kernelParam2=p2, kernelParam3=p3)
+        assert c_nat.shape == (n // 32, m // 16, 4, 16, 8)
+        c_rm = mlk.gemm_layoutAB_ContinuousC_wapper(a, b_nat, n, m, k, kernelParam1=p1, kernelParam2=p2,
+                                                    kernelParam3=p3)
+        assert torch.equal(mlk.reLayoutC(c_nat), c_rm)
+        # layout-C of the result is layout-B of the row-major result
+        assert np.array_equal(bits(c_nat.cpu()), layouts.pack_layout_c(bits(c_rm.cpu())))
+        c_a = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, kernelParam1=p1, kernelParam2=p2, kernelParam3=p3)
+        assert torch.equal(c_a, c_rm)
+        assert_close(c_rm, ogemm.linear_expected(w, b), RTOL, ATOL, "native chain")
+
+
+def test_native_chain_config(mlk):
+    n = k = 8192
+    m = 32
+    w = randn((n, k), torch.bfloat16, 0.02, 2025)
+    b = randn((m, k), torch.bfloat16, 1.0, 2026)
+    a = pack_a(w).cuda()
+    b_nat = mlk.layoutB(b.cuda())
+    c_nat = mlk.gemm_layoutABC(a, b_nat)
+    c = mlk.reLayoutC(c_nat)
+    assert_close(c, ogemm.linear_expected(w, b), RTOL, ATOL, "ABC 8192")
+    # chain a second product on the native output: C1 is the layout-B operand of the next layer
+    w2 = randn((256, n), torch.bfloat16, 0.02, 2027)
+    c2 = mlk.reLayoutC(mlk.gemm_layoutABC(pack_a(w2).cuda(), c_nat))
+    assert_close(c2, ogemm.linear_expected(w2, c.cpu()), RTOL, ATOL, "chained")
+
+
+@pytest.mark.parametrize("m", [1, 4, 16, 33])
+@pytest.mark.parametrize("scaled", [False, True])
+def test_gemm_soft_fp8(mlk, m, scaled):
+    n, k = 1024, 2048
+    codes = fp8_codes((n, k), 2025)
+    b = randn((m, k), torch.bfloat16, 1.0, 2026)
+    g = torch.Generator().manual_seed(3)
+    scale = (torch.rand((n // 128, k // 128), generator=g) * 0.02 + 0.001).float() if scaled else \
+        torch.ones((n // 128, k // 128))
+    c = mlk.gemm_layoutA_soft_fp8(pack_a(codes).cuda(), scale.cuda(), b.cuda())
+    assert_close(c, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), b), RTOL, ATOL, "soft-fp8 gemm")
+    c2 = mlk.gemm_layoutA_linear(pack_a(codes).cuda(), b.cuda(), scale_matrix=scale.cuda())
+    assert torch.equal(c, c2)
+
+
+@pytest.mark.parametrize("m", [4, 16])
+def test_gemm_soft_fp8_config(mlk, m):
+    n, k = 28672, 8192
+    codes = fp8_codes((n, k), 2025)
+    b = randn((m, k), torch.bfloat16, 1.0, 2026)
+    scale = torch.ones((n // 128, k // 128))
+    c = mlk.gemm_layoutA_soft_fp8(pack_a(codes).cuda(), scale.cuda(), b.cuda())
+    # float64 product in row chunks to bound host memory
+    from oracle import softfp8
+    got = c.cpu()
+    for r0 in range(0, n, 4096):
+        wchunk = softfp8.dequant_weight_f32(codes[r0:r0 + 4096].numpy(), None)
+        assert_close(got[:, r0:r0 + 4096], ogemm.linear_expected(wchunk, b), RTOL, ATOL, "soft-fp8 config")
+
+
+def test_gemm_errors(mlk):
+    a = torch.zeros(8, 16, 16, 8, dtype=torch.bfloat16, device="cuda")   # 128 x 128
+    b = torch.zeros(16, 128, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="same k"):
+        mlk.gemm_layoutA(a, torch.zeros(16, 256, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(RuntimeError, match="2D"):
+        mlk.gemm_layoutA(a, b.view(1, 16, 128))
+    with pytest.raises(RuntimeError, match="m % 128"):
+        mlk.gemm_layoutA(torch.zeros(4, 16, 16, 8, dtype=torch.bfloat16, device="cuda"), b)
+    with pytest.raises(RuntimeError, match="5D"):
+        mlk.gemm_layoutABC(a, b)
+    with pytest.raises(RuntimeError, match="data type"):
+        mlk.gemm_layoutA(a, b.half())
+    assert mlk.gemm_layoutA(a, b).shape == (16, 128)

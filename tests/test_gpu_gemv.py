@@ -1,0 +1,113 @@
+"""GPU parity: GeMV over layout-A weights against the oracle (float64 product on the
+un-packed weights), rtol = atol = 1e-2, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gemm as ogemm, softfp8
+from helpers import randn, pack_a, fp8_codes, assert_close
+
+pytestmark = pytest.mark.gpu
+
+RTOL = ATOL = 1e-2
+
+
+@pytest.mark.parametrize("n,k", [(16, 32), (4096, 4096), (1024, 14336), (11008, 4096), (160, 28672)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gemv_16bit(mlk, n, k, dtype):
+    w = randn((n, k), dtype, 0.02, 2025)
+    x = randn((1, k), dtype, 1.0, 2026)
+    y = mlk.gemv_layoutA(pack_a(w).cuda(), x.cuda())
+    assert y.shape == (1, n) and y.dtype == dtype
+    assert_close(y, ogemm.linear_expected(w, x), RTOL, ATOL, "gemv")
+
+
+@pytest.mark.parametrize("block,p1,p2", [(64, 1, 1), (256, 1, 4), (256, 2, 2), (256, 4, 8), (512, 2, 6),
+                                         (1024, 1, 4), (1024, 16, 2)])
+def test_gemv_launch_parameters(mlk, block, p1, p2):
+    n, k = 2048, 4096
+    w = randn((n, k), torch.bfloat16, 0.02, 1)
+    x = randn((1, k), torch.bfloat16, 1.0, 2)
+    y = mlk.gemv_layoutA_wapper(pack_a(w).cuda(), x.cuda(), n, k, blockDimX=block, kernelId=1, kernelParam1=p1,
+                                kernelParam2=p2)
+    assert_close(y, ogemm.linear_expected(w, x), RTOL, ATOL, "gemv params")
+
+
+def test_gemv_alpha_bias_and_special_cases(mlk):
+    n, k = 256, 512
+    w = randn((n, k), torch.bfloat16, 0.05, 3)
+    x = randn((1, k), torch.bfloat16, 1.0, 4)
+    bias = randn((1, n), torch.bfloat16, 1.0, 5)
+    a = pack_a(w).cuda()
+    y = mlk.gemv_layoutA(a, x.cuda(), alpha=0.5, bias=bias.cuda())
+    assert_close(y, ogemm.linear_expected(w, x, 0.5, bias), RTOL, ATOL, "alpha+bias")
+    # alpha = 0 leaves the bias exactly
+    y0 = mlk.gemv_layoutA(a, x.cuda(), alpha=0.0, bias=bias.cuda())
+    assert torch.equal(y0.cpu(), bias)
+    # identity weights copy x exactly
+    eye = torch.eye(512, dtype=torch.bfloat16)
+    yi = mlk.gemv_layoutA(pack_a(eye).cuda(), x.cuda())
+    assert torch.equal(yi.cpu(), x)
+    with pytest.raises(RuntimeError, match="beta"):
+        mlk.gemv_layoutA(a, x.cuda(), beta=1.0)
+
+
+def test_gemv_is_deterministic(mlk):
+    n, k = 4096, 4096
+    a = pack_a(randn((n, k), torch.bfloat16, 0.02, 7)).cuda()
+    x = randn((1, k), torch.bfloat16, 1.0, 8).cuda()
+    y1 = mlk.gemv_layoutA(a, x)
+    y2 = mlk.gemv_layoutA(a, x)
+    assert torch.equal(y1, y2)
+
+
+@pytest.mark.parametrize("n,k", [(128, 128), (4096, 4096), (28672, 8192), (2112, 7168)])
+@pytest.mark.parametrize("scaled", [False, True])
+def test_gemv_soft_fp8(mlk, n, k, scaled):
+    codes = fp8_codes((n, k), 2025)
+    x = randn((1, k), torch.bfloat16, 1.0, 2026)
+    scale = None
+    if scaled:
+        g = torch.Generator().manual_seed(9)
+        scale = (torch.rand(((n + 127) // 128, (k + 127) // 128), generator=g) * 0.02 + 0.001).float()
+    y = mlk.gemv_layoutA(pack_a(codes).cuda(), x.cuda(), scale_matrix=None if scale is None else scale.cuda())
+    want = ogemm.softfp8_linear_expected(codes.numpy(), None if scale is None else scale.numpy(), x)
+    assert_close(y, want, RTOL, ATOL, "soft-fp8 gemv")
+
+
+def test_gemv_soft_fp8_all_codes_exact(mlk):
+    """Every finite e4m3 code, one per weight row, against the oracle's widening: with a one-hot x
+    the output is the dequantised weight itself, so the comparison is bit-exact."""
+    k = 64
+    codes = torch.tensor([c for c in range(256) if c not in (0x7F, 0xFF)] + [0, 0], dtype=torch.uint8)  # 256 rows
+    w = torch.zeros((256, k), dtype=torch.uint8)
+    w[:, 5] = codes
+    x = torch.zeros((1, k), dtype=torch.bfloat16)
+    x[0, 5] = 1.0
+    for s in (1.0, 0.37, 1.0 / 448.0):
+        scale = torch.full((2, 1), s, dtype=torch.float32)
+        y = mlk.gemv_layoutA(pack_a(w).cuda(), x.cuda(), scale_matrix=scale.cuda())
+        want = softfp8.bf16_bits_to_f32(softfp8.dequant_bf16_bits(codes.numpy(), np.float32(s)))
+        got = y.cpu().float().numpy().reshape(-1)
+        assert np.array_equal(got, want)  # values, so that -0 (code 0x80) compares equal to the +0 a sum yields
+
+
+def test_gemv_rows_2_to_4(mlk):
+    n, k = 512, 1024
+    w = randn((n, k), torch.float16, 0.02, 1)
+    for m in (2, 3, 4):
+        x = randn((m, k), torch.float16, 1.0, 10 + m)
+        y = mlk.gemv_layoutA_wapper(pack_a(w).cuda(), x.cuda(), n, k, blockDimX=256, kernelParam1=1, kernelParam2=4)
+        assert_close(y, ogemm.linear_expected(w, x), RTOL, ATOL, "gemv M=%d" % m)
+
+
+def test_gemv_errors(mlk):
+    a = torch.zeros(2, 4, 16, 8, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="vector"):
+        mlk.gemv_layoutA(a, torch.zeros(2, 32, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(RuntimeError, match="same k"):
+        mlk.gemv_layoutA(a, torch.zeros(1, 64, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(RuntimeError, match="4D"):
+        mlk.gemv_layoutA(a.view(2, 4, 128), torch.zeros(1, 32, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(RuntimeError, match="data type"):
+        mlk.gemv_layoutA(a, torch.zeros(1, 32, dtype=torch.float16, device="cuda"))

@@ -1,0 +1,72 @@
+"""GPU parity: relayout kernels against the oracle, bit-exact, through the C ABI."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import layouts
+from helpers import bits
+
+pytestmark = pytest.mark.gpu
+
+
+def _bits16(shape, seed):
+    rng = np.random.default_rng(seed)
+    return torch.from_numpy(rng.integers(-32768, 32767, size=shape, dtype=np.int16, endpoint=True))
+
+
+@pytest.mark.parametrize("n,k", [(16, 32), (128, 256), (4096, 4096), (11008, 4096)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_pack_unpack_layout_a(mlk, n, k, dtype):
+    w = _bits16((n, k), n + k).view(dtype)
+    nat = mlk.pack_layout_a(w.cuda())
+    assert nat.shape == (n // 16, k // 8, 16, 8)
+    assert np.array_equal(bits(nat.cpu()), layouts.pack_layout_a(bits(w)))
+    assert torch.equal(mlk.unpack_layout_a(nat).view(torch.int16).cpu(), w.view(torch.int16))
+
+
+def test_pack_layout_a_bytes_and_batch(mlk):
+    rng = np.random.default_rng(5)
+    w = torch.from_numpy(rng.integers(0, 255, size=(3, 64, 128), dtype=np.uint8, endpoint=True))
+    nat = mlk.pack_layout_a(w.cuda()).cpu().numpy()
+    for e in range(3):
+        assert np.array_equal(nat[e], layouts.pack_layout_a(w[e].numpy()))
+    assert torch.equal(mlk.unpack_layout_a(torch.from_numpy(nat).cuda()).cpu(), w)
+
+
+@pytest.mark.parametrize("m,k", [(16, 32), (32, 8192), (64, 4096), (256, 4096), (2048, 256)])
+def test_layout_b(mlk, m, k):
+    b = _bits16((m, k), m * 7 + k).view(torch.bfloat16)
+    nat = mlk.layoutB(b.cuda())
+    assert nat.shape == (k // 32, m // 16, 4, 16, 8)
+    assert np.array_equal(bits(nat.cpu()), layouts.pack_layout_b(bits(b)))
+    # layout-C is layout-B with k := m, so reLayoutC inverts layoutB
+    assert torch.equal(mlk.reLayoutC(nat).view(torch.int16).cpu(), b.view(torch.int16))
+
+
+@pytest.mark.parametrize("m,n", [(16, 32), (32, 8192), (1712, 128)])  # 1712/16 = 107 > 104 token groups
+def test_re_layout_c(mlk, m, n):
+    c = _bits16((m, n), m + n).view(torch.float16)
+    c_nat = torch.from_numpy(layouts.pack_layout_c(bits(c))).view(torch.float16)
+    out = mlk.reLayoutC(c_nat.cuda())
+    assert out.shape == (m, n)
+    assert torch.equal(out.view(torch.int16).cpu(), c.view(torch.int16))
+
+
+@pytest.mark.parametrize("shape", [(256, 256), (100, 36), (3, 512, 256), (28672, 8192)])
+def test_fp8_weight_repack(mlk, shape):
+    rng = np.random.default_rng(11)
+    w = torch.from_numpy(rng.integers(0, 255, size=shape, dtype=np.uint8, endpoint=True))
+    out = mlk.fp8_weight_repack(w.cuda())
+    assert np.array_equal(out.cpu().numpy(), layouts.fp8_weight_repack(w.numpy()))
+    assert torch.equal(mlk.fp8_weight_repack(out).cpu(), w)  # involution
+
+
+def test_relayout_errors(mlk):
+    with pytest.raises(RuntimeError, match="multiple of 16"):
+        mlk.layoutB(torch.zeros(8, 32, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(RuntimeError, match="multiple of 32"):
+        mlk.layoutB(torch.zeros(16, 48, dtype=torch.bfloat16, device="cuda"))
+    with pytest.raises(RuntimeError, match="CUDA"):
+        mlk.layoutB(torch.zeros(16, 32, dtype=torch.bfloat16))
+    empty = mlk.layoutB(torch.zeros(0, 32, dtype=torch.bfloat16, device="cuda"))
+    assert empty.shape == (1, 0, 4, 16, 8)
