@@ -153,23 +153,25 @@ int mlk_moe_align_tokens(const int32_t *topk_ids, int n_pairs, int n_experts, in
                          const int32_t *experts_map, int32_t *sorted_token_ids, int32_t *cumsum_buffer,
                          int32_t *padded_num_blocks, int32_t *experts_ids, void *stream);
 
-/* Expert compute on an aligned batch: grouped gate/up GeMM with SiLU(gate)*up,
- * grouped down GeMM, routing-weighted sum back into token order.  Replaces both
- * overloads of `fused_experts_compute`,
- * csrc/moe_kernels/fused_experts_compute.cu:50-296 (ffi.cu:112-143).
+/* Expert compute from a routing decision: token -> expert-block alignment, grouped
+ * gate/up GeMM with SiLU(gate)*up, grouped down GeMM, routing-weighted sum back
+ * into token order.  Replaces both overloads of `fused_experts_compute`,
+ * csrc/moe_kernels/fused_experts_compute.cu:50-296 (ffi.cu:112-143), which run
+ * the alignment themselves (:6-48) before the three compute kernels.
  *   w1 [E, 2I, H] and w2 [E, H, I], each expert slab in layout-A; w_kind
  *   MLK_F16 / MLK_BF16 (= x_kind) or MLK_FP8_E4M3 with x_kind MLK_BF16 and fp32
- *   scales w1_scale [E, 2I/128, H/128], w2_scale [E, H/128, I/128]
- *   x [T, H], topk_weights [T*K] of x_kind, y [T, H] of x_kind (overwritten)
- *   sorted_token_ids / padded_num_blocks / experts_ids from mlk_moe_align_tokens
- *   workspace: at least mlk_moe_workspace_bytes() bytes of device scratch.
- * H % 128 == 0, I % 128 == 0. */
+ *   scales w1_scale [E, 2I/128, H/128], w2_scale [E, H/128, I/128] (NULL = 1)
+ *   x [T, H], topk_ids int32 [T*K], topk_weights [T*K] of x_kind,
+ *   experts_map int32 [E_global] or NULL (-1 drops the pair),
+ *   y [T, H] of x_kind (overwritten; needs no zero fill)
+ *   workspace: at least mlk_moe_workspace_bytes() bytes of device scratch
+ *   (alignment tables and the SiLU intermediate); contents are not preserved.
+ * H % 128 == 0, I % 128 == 0, E <= 256.  Tokens are processed in passes of 256. */
 int mlk_fused_experts_compute(const void *w1, const void *w2, const void *x, int n_tokens, int n_experts,
-                              int topk, int hidden, int inter, int w_kind, int x_kind,
-                              const void *topk_weights, const int32_t *sorted_token_ids,
-                              const int32_t *padded_num_blocks, const int32_t *experts_ids,
-                              const float *w1_scale, const float *w2_scale, void *y, void *workspace,
-                              size_t workspace_bytes, void *stream);
+                              int topk, int hidden, int inter, int w_kind, int x_kind, const int32_t *topk_ids,
+                              const void *topk_weights, const int32_t *experts_map, const float *w1_scale,
+                              const float *w2_scale, void *y, void *workspace, size_t workspace_bytes,
+                              void *stream);
 size_t mlk_moe_workspace_bytes(int n_tokens, int n_experts, int topk, int hidden, int inter);
 
 #ifdef __cplusplus

@@ -35,7 +35,7 @@ SIGNATURES = {
                                      c_void_p, c_void_p]),
     "mlk_fused_experts_compute": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                           c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
-                                          c_void_p, c_void_p, c_size_t, c_void_p]),
+                                          c_void_p, c_size_t, c_void_p]),
     "mlk_moe_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
 }
 

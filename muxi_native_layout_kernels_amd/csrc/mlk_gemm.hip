@@ -41,17 +41,13 @@ struct GemmArgs {
     float alpha;
 };
 
-// Most threads a workgroup may have for a given accumulator tile count, so that the
-// register file holds the accumulators plus the prefetch ring without spilling.
-__host__ __device__ constexpr int max_threads_for(int ntile) { return ntile <= 4 ? 1024 : (ntile <= 8 ? 512 : 256); }
-
 template <class T, bool FP8, int CB, int R, int BMODE, int CMODE, int U>
-__global__ void __launch_bounds__(max_threads_for(R *CB)) gemm_wave_kernel(GemmArgs p) {
+__global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel(GemmArgs p) {
     extern __shared__ f32x4 red[];  // [WK][R*CB][64]
     __shared__ int s_last;
 
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, kept scalar
     const int q = lane >> 4, r16 = lane & 15;
     const int sk = blockIdx.x % p.SK;
     const int rt = blockIdx.x / p.SK;
@@ -107,26 +103,57 @@ __global__ void __launch_bounds__(max_threads_for(R *CB)) gemm_wave_kernel(GemmA
             else bf[slot][cb] = u32x4{0u, 0u, 0u, 0u};
         }
     };
+    auto consume = [&](int slot) {
+        u32x4 a[R], b[CB];
 #pragma unroll
-    for (int u = 0; u < U; ++u)
-        if (u < nt) issue(u, tbeg + wave + u * p.WK);
+        for (int r = 0; r < R; ++r) a[r] = weight_operand<FP8>(wf[slot][r], FP8 ? sc[slot][r] : 1.f);
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) b[cb] = bf[slot][cb];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) acc[r][cb] = T::mfma(a[r], b[cb], acc[r][cb]);
+    };
+    // The wave visits its k tiles in a rotated order that differs from row tile to row tile:
+    // workgroups that run side by side then read different parts of the (small, shared)
+    // activation matrix at any moment instead of all hitting the same cache lines.
+    int jcur = nt > 0 ? (int)(((unsigned)rt * 2654435761u >> 7) % (unsigned)nt) : 0;
+    auto next_tile = [&]() {
+        int t = tbeg + wave + jcur * p.WK;
+        jcur = (jcur + 1 == nt) ? 0 : jcur + 1;
+        return t;
+    };
 
-    for (int i = 0; i < nt; i += U) {
+    // Register ring of U k-tiles; the steady-state loop is branch-free so the loads stay
+    // U tiles deep in flight.
+    if (nt >= U) {
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (i + u < nt) {
-                u32x4 a[R], b[CB];
+        for (int u = 0; u < U; ++u) issue(u, next_tile());
+        int i = 0;
+        for (; i + 2 * U <= nt; i += U) {
 #pragma unroll
-                for (int r = 0; r < R; ++r) a[r] = weight_operand<FP8>(wf[u][r], FP8 ? sc[u][r] : 1.f);
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb) b[cb] = bf[u][cb];
-                if (i + u + U < nt) issue(u, tbeg + wave + (i + u + U) * p.WK);
-#pragma unroll
-                for (int r = 0; r < R; ++r)
-#pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) acc[r][cb] = T::mfma(a[r], b[cb], acc[r][cb]);
+            for (int u = 0; u < U; ++u) {
+                consume(u);
+                issue(u, next_tile());
+                __builtin_amdgcn_sched_barrier(0);  // keep each refill right behind its consume
             }
         }
+        const int rem = nt - i - U;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            consume(u);
+            if (u < rem) issue(u, next_tile());
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < rem) consume(u);
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < nt) issue(u, next_tile());
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < nt) consume(u);
     }
 
     constexpr int NTILE = R * CB;
@@ -205,7 +232,7 @@ template <class T, bool FP8, int CB, int R, int BMODE, int CMODE>
 static int launch(const GemmArgs &p, hipStream_t s) {
     constexpr int U = (R * CB >= 8) ? 2 : ((R * CB >= 4) ? 3 : 4);
     GemmArgs q = p;
-    while (q.WK * 64 > max_threads_for(R * CB) || (size_t)q.WK * R * CB * 1024 > 64 * 1024) q.WK >>= 1;
+    while (q.WK * 64 > max_threads_for_tiles(R * CB) || (size_t)q.WK * R * CB * 1024 > 64 * 1024) q.WK >>= 1;
     int row_tiles = (q.N / 16) / R;
     int grid = row_tiles * q.SK;
     size_t lds = q.WK > 1 ? (size_t)q.WK * R * CB * 1024 : 0;

@@ -13,6 +13,12 @@
 
 namespace mlk {
 
+// Most threads a workgroup may have for a given number of 16x16 accumulator tiles per wave,
+// so that the register file holds the accumulators plus the prefetch ring without spilling.
+__host__ __device__ constexpr int max_threads_for_tiles(int ntile) {
+    return ntile <= 4 ? 1024 : (ntile <= 8 ? 512 : 256);
+}
+
 // One k-tile (32 k) of weights for one row group, as an MFMA operand.
 template <bool FP8>
 struct WeightFrag {

@@ -30,7 +30,7 @@ __global__ void __launch_bounds__(1024)
 
     constexpr int TK = FP8 ? 64 : 32;             // k covered by one 1 KiB tile
     const int lane = threadIdx.x & 63;
-    const int wave = threadIdx.x >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, kept scalar
     const int rg_local = wave / WK;
     const int ks = wave - rg_local * WK;
     const int rg = blockIdx.x * G + rg_local;
@@ -59,15 +59,52 @@ __global__ void __launch_bounds__(1024)
         const int nt = (active && ks < tiles_here) ? (tiles_here - ks + WK - 1) / WK : 0;
         const u32x4 *ap = arow + (size_t)(t0 + ks) * 64;
 
-        // start the weight stream before touching the activations
+        // Register ring of U tiles.  The steady-state loop is branch-free so that the
+        // loads stay U deep in flight (the waits become vmcnt(U-1)).
         u32x4 buf[U];
         float sc[U];
+        auto issue = [&](int u, int j) {          // j = index among this wave's tiles in the window
+            buf[u] = ld_stream_u32x4(ap + (size_t)j * stride);
+            if (FP8) sc[u] = scale ? scale[(rg >> 3) * scale_cols + ((t0 + ks + j * WK) >> 1)] : 1.f;
+        };
+        auto consume = [&](int u, int j) {
+            u32x4 cur = buf[u];
+            const int xg = (ks + j * WK) * (TK / 8) + oct;   // granule of 8 activations
+            if (FP8) {
+                float s = sc[u];
+                uint32_t w0[4], w1[4];
+                fp8x4_to_bf16x4(cur[0], s, w0[0], w0[1]);
+                fp8x4_to_bf16x4(cur[1], s, w0[2], w0[3]);
+                fp8x4_to_bf16x4(cur[2], s, w1[0], w1[1]);
+                fp8x4_to_bf16x4(cur[3], s, w1[2], w1[3]);
 #pragma unroll
-        for (int u = 0; u < U; ++u) {
-            if (u < nt) {
-                buf[u] = ld_stream_u32x4(ap + (size_t)u * stride);
-                if (FP8) sc[u] = scale ? scale[(rg >> 3) * scale_cols + ((t0 + ks + u * WK) >> 1)] : 1.f;
+                for (int m = 0; m < M; ++m) {
+                    u32x4 xv = xs[m * (KC >> 3) + xg];
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) {
+                        acc[0][m] = T::dot2(w0[d], xv[d], acc[0][m]);
+                        acc[FP8 ? 1 : 0][m] = T::dot2(w1[d], xv[d], acc[FP8 ? 1 : 0][m]);
+                    }
+                }
+            } else {
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    u32x4 xv = xs[m * (KC >> 3) + xg];
+#pragma unroll
+                    for (int d = 0; d < 4; ++d) acc[0][m] = T::dot2(cur[d], xv[d], acc[0][m]);
+                }
             }
+        };
+
+        // start the weight stream before touching the activations
+        const bool full = nt >= U;
+        if (full) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) issue(u, u);
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < nt) issue(u, u);
         }
 
         if (kc0 > 0) __syncthreads();             // everyone is done with the previous window
@@ -78,43 +115,29 @@ __global__ void __launch_bounds__(1024)
         }
         __syncthreads();
 
-        for (int i = 0; i < nt; i += U) {
+        if (full) {
+            int i = 0;
+            for (; i + 2 * U <= nt; i += U) {
 #pragma unroll
-            for (int u = 0; u < U; ++u) {
-                if (i + u < nt) {
-                    u32x4 cur = buf[u];
-                    float s = FP8 ? sc[u] : 1.f;
-                    const int kt = ks + (i + u) * WK;             // tile index inside the window
-                    if (i + u + U < nt) {
-                        buf[u] = ld_stream_u32x4(ap + (size_t)(i + u + U) * stride);
-                        if (FP8) sc[u] = scale ? scale[(rg >> 3) * scale_cols + ((t0 + kt + U * WK) >> 1)] : 1.f;
-                    }
-                    const int xg = kt * (TK / 8) + oct;            // granule of 8 activations
-                    if (FP8) {
-                        uint32_t w0[4], w1[4];
-                        fp8x4_to_bf16x4(cur[0], s, w0[0], w0[1]);
-                        fp8x4_to_bf16x4(cur[1], s, w0[2], w0[3]);
-                        fp8x4_to_bf16x4(cur[2], s, w1[0], w1[1]);
-                        fp8x4_to_bf16x4(cur[3], s, w1[2], w1[3]);
-#pragma unroll
-                        for (int m = 0; m < M; ++m) {
-                            u32x4 xv = xs[m * (KC >> 3) + xg];
-#pragma unroll
-                            for (int d = 0; d < 4; ++d) {
-                                acc[0][m] = T::dot2(w0[d], xv[d], acc[0][m]);
-                                acc[FP8 ? 1 : 0][m] = T::dot2(w1[d], xv[d], acc[FP8 ? 1 : 0][m]);
-                            }
-                        }
-                    } else {
-#pragma unroll
-                        for (int m = 0; m < M; ++m) {
-                            u32x4 xv = xs[m * (KC >> 3) + xg];
-#pragma unroll
-                            for (int d = 0; d < 4; ++d) acc[0][m] = T::dot2(cur[d], xv[d], acc[0][m]);
-                        }
-                    }
+                for (int u = 0; u < U; ++u) {
+                    consume(u, i + u);
+                    issue(u, i + U + u);
+                    __builtin_amdgcn_sched_barrier(0);  // keep each refill right behind its consume
                 }
             }
+            const int rem = nt - i - U;           // 0 .. U-1 tiles still to be fetched
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                consume(u, i + u);
+                if (u < rem) issue(u, i + U + u);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < rem) consume(u, i + U + u);
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < nt) consume(u, u);
         }
     }
 

@@ -1,8 +1,719 @@
-#include "mlk_common.cuh"
+// Fused MoE for gfx950: router, token -> expert-block alignment and the two
+// grouped GeMMs over per-expert layout-A weight slabs.
+//
+//   router      one wave per token: scores (softmax / sigmoid), optional
+//               selection bias, grouped selection, iterative arg-max top-K with
+//               ties to the lower id, optional renormalisation
+//   align       one workgroup: per-expert counts, padding to 16-slot blocks,
+//               prefix sum, block owners, and a stable scatter (ascending flat
+//               pair index inside each expert) - deterministic, no atomics on
+//               the output positions.  It also writes the task list the GeMMs
+//               walk: (expert, first block, number of blocks <= CB).
+//   gate/up     grid (row tile, task): streams the gate rows and the matching
+//               up rows of W1[expert] once, gathers the task's tokens as MFMA
+//               activation fragments, and stores T(silu(gate) * up) in
+//               layout-B so the second GeMM reads it with coalesced loads
+//   down        grid (row tile): walks ALL tasks, streams W2[expert] rows, and
+//               adds routing weight * product into an fp32 [tokens x rows] tile
+//               in LDS; one rounding to T at the end.  This is the weighted
+//               un-permute: no atomics, no intermediate [pairs, H] buffer, fixed
+//               summation order.
+//
+// Algorithmic traffic per layer: active experts * 3*I*H*sizeof(W) (+ scales)
+// + 2*T*H*2 + T*E*2 bytes; the SiLU intermediate (T*K*I*2 bytes, written and
+// read once) stays in L2 / Infinity Cache for decode-sized T.
+#include "mlk_gemm_tile.cuh"
+
+namespace mlk {
+
+constexpr int kMaxExperts = 256;
+constexpr int kMaxTopK = 32;
+constexpr int kMoeChunk = 256;     // tokens per expert-compute pass
+
+// ------------------------------------------------------------------ router
+template <class T>
+__global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__ logits, int n_tokens, int E,
+                                                    int n_groups, int topk_groups, int topk, int score_fun,
+                                                    const uint16_t *__restrict__ bias, int renorm,
+                                                    int32_t *__restrict__ ids, uint16_t *__restrict__ weights) {
+    __shared__ double ex[kMaxExperts];     // logits, then exp(x - max)
+    __shared__ float prob[kMaxExperts];    // un-biased score rounded to T
+    __shared__ float sel[kMaxExperts];     // selection score rounded to T
+    __shared__ float gscore[kMaxExperts];
+    __shared__ int keep[kMaxExperts];
+    __shared__ double s_sum;
+    __shared__ int pick_id[kMaxTopK];
+    __shared__ float pick_w[kMaxTopK];
+
+    const int tok = blockIdx.x;
+    const int lane = threadIdx.x;
+    const uint16_t *row = logits + (size_t)tok * E;
+    auto round_T = [](float v) { return T::to_f32(T::from_f32(v)); };
+
+    // scores: exp, the index-order sum and the division in float64, one rounding to fp32, one to T
+    double mx = -1.0e300;
+    for (int j = lane; j < E; j += 64) {
+        double v = (double)T::to_f32(row[j]);
+        ex[j] = v;
+        mx = fmax(mx, v);
+    }
+    for (int m = 32; m >= 1; m >>= 1) {
+        double o = __shfl_xor(mx, m);
+        mx = fmax(mx, o);
+    }
+    if (score_fun == 0) {
+        for (int j = lane; j < E; j += 64) ex[j] = exp(ex[j] - mx);
+        __syncthreads();
+        if (lane == 0) {
+            double s = 0.0;
+            for (int j = 0; j < E; ++j) s += ex[j];
+            s_sum = s;
+        }
+        __syncthreads();
+        const double s = s_sum;
+        for (int j = lane; j < E; j += 64) prob[j] = round_T((float)(ex[j] / s));
+    } else {
+        for (int j = lane; j < E; j += 64) prob[j] = round_T((float)(1.0 / (1.0 + exp(-ex[j]))));
+    }
+    for (int j = lane; j < E; j += 64) sel[j] = bias ? round_T(prob[j] + T::to_f32(bias[j])) : prob[j];
+    __syncthreads();
+
+    // group scores: max of the group, or the T-sum of its two largest positive scores with a bias
+    const int per_group = E / n_groups;
+    for (int g = lane; g < n_groups; g += 64) {
+        const float *seg = sel + g * per_group;
+        float score;
+        if (!bias) {
+            score = 0.f;
+            for (int j = 0; j < per_group; ++j) score = seg[j] > score ? seg[j] : score;
+        } else {
+            float a = 0.f, b = 0.f;  // largest, second largest positive
+            for (int j = 0; j < per_group; ++j) {
+                float v = seg[j];
+                if (v > a) { b = a; a = v; }
+                else if (v > b) b = v;
+            }
+            score = 0.f;
+            if (a > 0.f) score = round_T(a + score);
+            if (b > 0.f) score = round_T(b + score);
+        }
+        gscore[g] = score;
+        keep[g] = 0;
+    }
+    __syncthreads();
+    if (lane == 0) {
+        for (int i = 0; i < topk_groups; ++i) {
+            int best = 0;
+            for (int g = 1; g < n_groups; ++g)
+                if (gscore[g] > gscore[best]) best = g;
+            keep[best] = 1;
+            gscore[best] = 0.f;
+        }
+    }
+    __syncthreads();
+    for (int j = lane; j < E; j += 64)
+        if (!keep[j / per_group]) { sel[j] = 0.f; prob[j] = 0.f; }
+    __syncthreads();
+
+    // K rounds of arg-max over the selection scores, ties to the lower id; a picked score becomes 0
+    for (int kk = 0; kk < topk; ++kk) {
+        float bv = sel[lane < E ? lane : 0];
+        int bi = lane < E ? lane : 0;
+        for (int j = lane + 64; j < E; j += 64)
+            if (sel[j] > bv) { bv = sel[j]; bi = j; }
+        if (lane >= E) { bv = -3.0e38f; bi = 0x7fffffff; }
+        for (int m = 32; m >= 1; m >>= 1) {
+            float ov = __shfl_xor(bv, m);
+            int oi = __shfl_xor(bi, m);
+            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        }
+        if (lane == 0) {
+            pick_id[kk] = bi;
+            pick_w[kk] = prob[bi];
+            sel[bi] = 0.f;
+        }
+        __syncthreads();
+    }
+
+    if (lane == 0) {
+        if (score_fun == 0) {
+            // the softmax variant returns its picks ordered by expert id
+            for (int a = 1; a < topk; ++a) {
+                int id = pick_id[a];
+                float w = pick_w[a];
+                int b = a - 1;
+                while (b >= 0 && pick_id[b] > id) {
+                    pick_id[b + 1] = pick_id[b];
+                    pick_w[b + 1] = pick_w[b];
+                    --b;
+                }
+                pick_id[b + 1] = id;
+                pick_w[b + 1] = w;
+            }
+        }
+        float denom = 1.f;
+        if (renorm) {
+            float s = 0.f;
+            for (int a = 0; a < topk; ++a) s += pick_w[a];
+            denom = round_T(s);
+        }
+        for (int a = 0; a < topk; ++a) {
+            ids[(size_t)tok * topk + a] = pick_id[a];
+            float w = renorm ? pick_w[a] / denom : pick_w[a];
+            weights[(size_t)tok * topk + a] = (uint16_t)T::from_f32(w);
+        }
+    }
+}
+
+// ------------------------------------------------------------------- align
+struct MoeTask {
+    int expert, block0, nblocks, pad;
+};
+
+__global__ void __launch_bounds__(1024) moe_align_kernel(const int32_t *__restrict__ topk_ids, int n_pairs, int E,
+                                                         const int32_t *__restrict__ experts_map,
+                                                         int32_t *__restrict__ sorted_ids,
+                                                         int32_t *__restrict__ cumsum_out,
+                                                         int32_t *__restrict__ padded_blocks,
+                                                         int32_t *__restrict__ experts_ids, int max_blocks,
+                                                         MoeTask *__restrict__ tasks, int32_t *__restrict__ n_tasks,
+                                                         int cb_max) {
+    constexpr int NW = 16;
+    __shared__ int cnt[NW][kMaxExperts];   // per-wave counts, then per-wave write cursors
+    __shared__ int start[kMaxExperts + 1]; // padded exclusive prefix
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int max_padded = n_pairs + E * 15;
+
+    for (int i = tid; i < NW * kMaxExperts; i += 1024) (&cnt[0][0])[i] = 0;
+    for (int i = tid; i < max_padded; i += 1024) sorted_ids[i] = n_pairs;   // sentinel everywhere
+    for (int i = tid; i < max_blocks; i += 1024) experts_ids[i] = 0;
+    __syncthreads();
+
+    // each wave owns a contiguous range of 64-pair tiles
+    const int n_tiles = (n_pairs + 63) >> 6;
+    const int tiles_per = (n_tiles + NW - 1) / NW;
+    const int t_beg = wave * tiles_per;
+    const int t_end = min(n_tiles, t_beg + tiles_per);
+    auto local_expert = [&](int i) -> int {
+        if (i >= n_pairs) return -1;
+        int e = topk_ids[i];
+        if (experts_map) e = experts_map[e];
+        return (e >= 0 && e < E) ? e : -1;
+    };
+    for (int t = t_beg; t < t_end; ++t) {
+        int e = local_expert(t * 64 + lane);
+        if (e >= 0) atomicAdd(&cnt[wave][e], 1);
+    }
+    __syncthreads();
+
+    // totals -> padded prefix (one thread; E <= 256) ; per-wave cursors
+    if (tid == 0) {
+        int run = 0, nt = 0;
+        for (int e = 0; e < E; ++e) {
+            int total = 0;
+            for (int w = 0; w < NW; ++w) total += cnt[w][e];
+            start[e] = run;
+            int nb = (total + 15) >> 4;
+            for (int b = 0; b < nb; ++b) experts_ids[(run >> 4) + b] = e;
+            if (tasks) {
+                for (int b = 0; b < nb; b += cb_max) {
+                    MoeTask tk;
+                    tk.expert = e;
+                    tk.block0 = (run >> 4) + b;
+                    tk.nblocks = min(cb_max, nb - b);
+                    tk.pad = 0;
+                    tasks[nt++] = tk;
+                }
+            }
+            run += nb << 4;
+            cumsum_out[e] = start[e] + total;          // where the reference's atomic cursor ends up
+        }
+        start[E] = run;
+        cumsum_out[E] = run;
+        padded_blocks[0] = run >> 4;
+        if (n_tasks) n_tasks[0] = nt;
+    }
+    __syncthreads();
+    for (int e = tid; e < E; e += 1024) {
+        int run = start[e];
+        for (int w = 0; w < NW; ++w) {
+            int c = cnt[w][e];
+            cnt[w][e] = run;
+            run += c;
+        }
+    }
+    __syncthreads();
+
+    // stable scatter: inside a 64-pair tile, lanes with the same expert are ranked by lane id
+    for (int t = t_beg; t < t_end; ++t) {
+        const int i = t * 64 + lane;
+        const int e = local_expert(i);
+        unsigned long long todo = __ballot(e >= 0);
+        int pos = -1;
+        while (todo) {
+            const int leader = __ffsll((long long)todo) - 1;
+            const int le = __shfl(e, leader);
+            const unsigned long long same = __ballot(e == le);
+            if (e == le) {
+                const unsigned long long below = same & ((1ull << lane) - 1ull);
+                pos = cnt[wave][le] + __popcll(below);
+            }
+            __builtin_amdgcn_wave_barrier();
+            if (lane == leader) cnt[wave][le] += __popcll(same);
+            __builtin_amdgcn_wave_barrier();
+            todo &= ~same;
+        }
+        if (pos >= 0) sorted_ids[pos] = i;
+    }
+}
+
+// ------------------------------------------------------------ grouped GeMMs
+struct MoeArgs {
+    const uint8_t *W1;        // [E][2I][H] layout-A slabs
+    const uint8_t *W2;        // [E][H][I]
+    const float *S1;          // [E][2I/128][H/128] or null
+    const float *S2;          // [E][H/128][I/128] or null
+    const uint16_t *X;        // [T][H]
+    uint16_t *Y;              // [T][H]
+    uint16_t *Hbuf;           // layout-B [I/32][SB][4][16][8]
+    const uint16_t *wts;      // [T*K]
+    const int32_t *sorted;    // [T*K + E*15]
+    const MoeTask *tasks;
+    const int32_t *n_tasks;
+    int T, K, H, I, SB, n_pairs, WK;
+};
+
+// gate/up projection with SiLU(gate) * up, one task per blockIdx.y
+template <class T, bool FP8, int CB, int P, int U>
+__global__ void __launch_bounds__(max_threads_for_tiles(2 * P * CB)) moe_gate_up_kernel(MoeArgs p) {
+    extern __shared__ f32x4 red[];  // [WK][2P*CB][64]
+    const int task = blockIdx.y;
+    if (task >= p.n_tasks[0]) return;
+    const MoeTask tk = p.tasks[task];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = lane >> 4, r16 = lane & 15;
+    const int g0 = blockIdx.x * P;
+    constexpr int WB = FP8 ? 1 : 2;
+    constexpr int R = 2 * P;                       // weight streams per wave: gate, up, gate, up ...
+    const int tiles_total = p.H >> 5;
+    const int groups_i = p.I >> 4;
+    const size_t slab = (size_t)2 * p.I * p.H * WB;
+    const int scale_cols = p.H >> 7;
+
+    const uint8_t *abase[R];
+    int srow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        int rg = (r & 1) * groups_i + g0 + (r >> 1);
+        abase[r] = p.W1 + (size_t)tk.expert * slab + (size_t)rg * p.H * 16 * WB;
+        srow[r] = (tk.expert * (2 * p.I >> 7) + (rg >> 3)) * scale_cols;
+    }
+    const uint16_t *bptr[CB];
+    bool bok[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        int id = p.n_pairs;
+        if (cb < tk.nblocks) id = p.sorted[(tk.block0 + cb) * 16 + r16];
+        bok[cb] = id < p.n_pairs;
+        bptr[cb] = p.X + (size_t)(bok[cb] ? id / p.K : 0) * p.H + q * 8;
+    }
+
+    f32x4 acc[R][CB];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int nt = (wave < tiles_total) ? (tiles_total - wave + p.WK - 1) / p.WK : 0;
+    WeightFrag<FP8> wf[U][R];
+    u32x4 bf[U][CB];
+    float sc[U][R];
+    auto issue = [&](int slot, int kt) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
+            if (FP8) sc[slot][r] = p.S1 ? p.S1[srow[r] + (kt >> 2)] : 1.f;
+        }
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            if (bok[cb]) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * 32);
+            else bf[slot][cb] = u32x4{0u, 0u, 0u, 0u};
+        }
+    };
+    auto consume = [&](int slot) {
+        u32x4 a[R], b[CB];
+#pragma unroll
+        for (int r = 0; r < R; ++r) a[r] = weight_operand<FP8>(wf[slot][r], FP8 ? sc[slot][r] : 1.f);
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) b[cb] = bf[slot][cb];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) acc[r][cb] = T::mfma(a[r], b[cb], acc[r][cb]);
+    };
+    int jcur = 0;
+    auto next_tile = [&]() { return wave + (jcur++) * p.WK; };
+    if (nt >= U) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) issue(u, next_tile());
+        int i = 0;
+        for (; i + 2 * U <= nt; i += U) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                consume(u);
+                issue(u, next_tile());
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        const int rem = nt - i - U;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            consume(u);
+            if (u < rem) issue(u, next_tile());
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < rem) consume(u);
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < nt) issue(u, next_tile());
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < nt) consume(u);
+    }
+
+    // fold the waves in wave order, then SiLU(gate) * up and the layout-B store
+    constexpr int NT = R * CB;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) red[(wave * NT + r * CB + cb) * 64 + lane] = acc[r][cb];
+    __syncthreads();
+    for (int j = wave; j < P * CB; j += p.WK) {
+        const int pr = j / CB, cb = j - pr * CB;
+        if (cb >= tk.nblocks) continue;
+        const int jg = (2 * pr) * CB + cb, ju = (2 * pr + 1) * CB + cb;
+        f32x4 g = red[jg * 64 + lane], u = red[ju * 64 + lane];
+        for (int w = 1; w < p.WK; ++w) {
+            g += red[(w * NT + jg) * 64 + lane];
+            u += red[(w * NT + ju) * 64 + lane];
+        }
+        float h[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) h[i] = g[i] / (1.f + __expf(-g[i])) * u[i];
+        const int n = (g0 + pr) * 16 + 4 * q;           // intermediate index = k of the down projection
+        const size_t off =
+            ((((size_t)(n >> 5) * p.SB + (tk.block0 + cb)) * 4 + ((n & 31) >> 3)) * 16 + r16) * 8 + (n & 7);
+        store4<T>(p.Hbuf + off, h[0], h[1], h[2], h[3]);
+    }
+}
+
+// down projection over all tasks, routing weights and the sum over a token's experts in LDS
+template <class T, bool FP8, int CB, int R, int U>
+__global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(MoeArgs p) {
+    extern __shared__ f32x4 red[];  // [WK][R*CB][64] then the fp32 output tile [T][16R]
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = lane >> 4, r16 = lane & 15;
+    const int rg0 = blockIdx.x * R;
+    constexpr int WB = FP8 ? 1 : 2;
+    constexpr int NT = R * CB;
+    const int tiles_total = p.I >> 5;
+    const size_t slab = (size_t)p.H * p.I * WB;
+    const int scale_cols = p.I >> 7;
+    float *ytile = reinterpret_cast<float *>(red + (size_t)p.WK * NT * 64);
+    const int yrows = 16 * R;
+
+    for (int i = threadIdx.x; i < p.T * yrows; i += blockDim.x) ytile[i] = 0.f;
+    __syncthreads();
+
+    const int n_tasks = p.n_tasks[0];
+    const int nt = (wave < tiles_total) ? (tiles_total - wave + p.WK - 1) / p.WK : 0;
+    for (int task = 0; task < n_tasks; ++task) {
+        const MoeTask tk = p.tasks[task];
+        const uint8_t *abase[R];
+        int srow[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            abase[r] = p.W2 + (size_t)tk.expert * slab + (size_t)(rg0 + r) * p.I * 16 * WB;
+            srow[r] = (tk.expert * (p.H >> 7) + ((rg0 + r) >> 3)) * scale_cols;
+        }
+        const uint16_t *bptr[CB];
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) bptr[cb] = p.Hbuf + ((size_t)(tk.block0 + cb) * 64 + lane) * 8;
+        const size_t bstep = (size_t)p.SB * 512;
+
+        f32x4 acc[R][CB];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        WeightFrag<FP8> wf[U][R];
+        u32x4 bf[U][CB];
+        float sc[U][R];
+        auto issue = [&](int slot, int kt) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
+                if (FP8) sc[slot][r] = p.S2 ? p.S2[srow[r] + (kt >> 2)] : 1.f;
+            }
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) {
+                if (cb < tk.nblocks) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * bstep);
+                else bf[slot][cb] = u32x4{0u, 0u, 0u, 0u};
+            }
+        };
+        auto consume = [&](int slot) {
+            u32x4 a[R], b[CB];
+#pragma unroll
+            for (int r = 0; r < R; ++r) a[r] = weight_operand<FP8>(wf[slot][r], FP8 ? sc[slot][r] : 1.f);
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) b[cb] = bf[slot][cb];
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) acc[r][cb] = T::mfma(a[r], b[cb], acc[r][cb]);
+        };
+        int jcur = 0;
+        auto next_tile = [&]() { return wave + (jcur++) * p.WK; };
+        if (nt >= U) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) issue(u, next_tile());
+            int i = 0;
+            for (; i + 2 * U <= nt; i += U) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    consume(u);
+                    issue(u, next_tile());
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
+            const int rem = nt - i - U;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                consume(u);
+                if (u < rem) issue(u, next_tile());
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < rem) consume(u);
+        } else {
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < nt) issue(u, next_tile());
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < nt) consume(u);
+        }
+
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) red[(wave * NT + r * CB + cb) * 64 + lane] = acc[r][cb];
+        __syncthreads();
+        for (int j = wave; j < NT; j += p.WK) {
+            const int r = j / CB, cb = j - r * CB;
+            if (cb >= tk.nblocks) continue;
+            const int id = p.sorted[(tk.block0 + cb) * 16 + r16];
+            if (id >= p.n_pairs) continue;
+            f32x4 v = red[j * 64 + lane];
+            for (int w = 1; w < p.WK; ++w) v += red[(w * NT + j) * 64 + lane];
+            const float wt = T::to_f32(p.wts[id]);
+            float *dst = ytile + (size_t)(id / p.K) * yrows + r * 16 + 4 * q;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) dst[i] += wt * v[i];
+        }
+        __syncthreads();
+    }
+
+    for (int i = threadIdx.x; i < p.T * yrows; i += blockDim.x) {
+        int tok = i / yrows, row = i - tok * yrows;
+        p.Y[(size_t)tok * p.H + rg0 * 16 + row] = (uint16_t)T::from_f32(ytile[i]);
+    }
+}
+
+// ----------------------------------------------------------- host-side glue
+struct MoeWorkspace {
+    MoeTask *tasks;
+    int32_t *n_tasks;
+    int32_t *sorted, *cumsum, *padded, *experts_ids;
+    uint16_t *hbuf;
+};
+
+static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+static size_t carve(uint8_t *base, int tc, int E, int K, int inter, MoeWorkspace *ws) {
+    const int n_pairs = tc * K;
+    const int max_padded = n_pairs + E * 15;
+    const int max_blocks = (max_padded + 15) / 16;
+    size_t off = 0;
+    auto take = [&](size_t bytes) {
+        uint8_t *ptr = base ? base + off : nullptr;
+        off = align_up(off + bytes, 256);
+        return ptr;
+    };
+    MoeWorkspace w;
+    w.tasks = (MoeTask *)take(sizeof(MoeTask) * (size_t)(max_blocks + 1));
+    w.n_tasks = (int32_t *)take(sizeof(int32_t));
+    w.sorted = (int32_t *)take(sizeof(int32_t) * (size_t)max_padded);
+    w.cumsum = (int32_t *)take(sizeof(int32_t) * (size_t)(E + 1));
+    w.padded = (int32_t *)take(sizeof(int32_t));
+    w.experts_ids = (int32_t *)take(sizeof(int32_t) * (size_t)max_blocks);
+    w.hbuf = (uint16_t *)take((size_t)inter * max_blocks * 16 * 2);
+    if (ws) *ws = w;
+    return off;
+}
+
+template <class T, bool FP8, int CB>
+static int launch_moe(const MoeArgs &a, int max_tasks, hipStream_t s) {
+    // gate/up: one (gate, up) pair of row groups per wave for CB >= 2, two pairs for CB == 1
+    constexpr int P = (CB == 1) ? 2 : 1;
+    constexpr int U1 = (2 * P * CB >= 8) ? 2 : 3;
+    MoeArgs g = a;
+    const int groups_i = a.I / 16;
+    g.WK = 4;
+    while (g.WK * 64 > max_threads_for_tiles(2 * P * CB)) g.WK >>= 1;
+    const int grid_x = groups_i / P;   // I % 128 == 0 so this is exact for P <= 8
+    size_t lds1 = (size_t)g.WK * 2 * P * CB * 1024;
+    moe_gate_up_kernel<T, FP8, CB, P, U1><<<dim3(grid_x, max_tasks), g.WK * 64, lds1, s>>>(g);
+    MLK_LAUNCH_CHECK();
+
+    constexpr int R = 1;
+    constexpr int U2 = (CB >= 4) ? 3 : 4;
+    MoeArgs d = a;
+    d.WK = 16;
+    while (d.WK > 1 && (d.WK * 64 > max_threads_for_tiles(R * CB) ||
+                        (size_t)d.WK * R * CB * 1024 + (size_t)a.T * 16 * R * 4 > 64 * 1024))
+        d.WK >>= 1;
+    size_t lds2 = (size_t)d.WK * R * CB * 1024 + (size_t)a.T * 16 * R * 4;
+    moe_down_kernel<T, FP8, CB, R, U2><<<a.H / 16 / R, d.WK * 64, lds2, s>>>(d);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+template <class T, bool FP8>
+static int launch_moe_cb(const MoeArgs &a, int cb, int max_tasks, hipStream_t s) {
+    switch (cb) {
+        case 1: return launch_moe<T, FP8, 1>(a, max_tasks, s);
+        case 2: return launch_moe<T, FP8, 2>(a, max_tasks, s);
+        case 3: return launch_moe<T, FP8, 3>(a, max_tasks, s);
+        default: return launch_moe<T, FP8, 4>(a, max_tasks, s);
+    }
+}
+
+}  // namespace mlk
+
 using namespace mlk;
-extern "C" {
-int mlk_fused_routing_gate(const void *, int, int, int, int, int, int, int, const void *, int, int32_t *, void *, void *) { return fail(MLK_ERR_INVALID, "not built yet"); }
-int mlk_moe_align_tokens(const int32_t *, int, int, int, const int32_t *, int32_t *, int32_t *, int32_t *, int32_t *, void *) { return fail(MLK_ERR_INVALID, "not built yet"); }
-int mlk_fused_experts_compute(const void *, const void *, const void *, int, int, int, int, int, int, int, const void *, const int32_t *, const int32_t *, const int32_t *, const float *, const float *, void *, void *, size_t, void *) { return fail(MLK_ERR_INVALID, "not built yet"); }
-size_t mlk_moe_workspace_bytes(int, int, int, int, int) { return 0; }
+
+extern "C" int mlk_fused_routing_gate(const void *logits, int x_kind, int score_fun, int n_tokens, int n_experts,
+                                      int n_groups, int topk_groups, int topk, const void *bias, int renormalize,
+                                      int32_t *ids, void *weights, void *stream) {
+    MLK_REQUIRE(x_kind == MLK_F16 || x_kind == MLK_BF16, "router: logits must be fp16 or bf16");
+    MLK_REQUIRE(score_fun == 0 || score_fun == 1, "router: score function must be 0 (softmax) or 1 (sigmoid)");
+    MLK_REQUIRE(n_tokens >= 0, "router: negative token count");
+    MLK_REQUIRE(n_experts >= 1 && n_experts <= kMaxExperts, "router: 1..256 experts");
+    MLK_REQUIRE(n_groups >= 1 && n_experts % n_groups == 0, "router: n_groups must divide the expert count");
+    MLK_REQUIRE(topk_groups >= 1 && topk_groups <= n_groups, "router: topk_groups must be in 1..n_groups");
+    MLK_REQUIRE(topk >= 1 && topk <= kMaxTopK && topk <= n_experts, "router: topk must be in 1..min(32, experts)");
+    if (n_tokens == 0) return MLK_OK;
+    MLK_REQUIRE(logits && ids && weights, "router: null pointer");
+    hipStream_t s = (hipStream_t)stream;
+    if (x_kind == MLK_F16)
+        router_kernel<F16><<<n_tokens, 64, 0, s>>>((const uint16_t *)logits, n_tokens, n_experts, n_groups,
+                                                   topk_groups, topk, score_fun, (const uint16_t *)bias, renormalize,
+                                                   ids, (uint16_t *)weights);
+    else
+        router_kernel<BF16><<<n_tokens, 64, 0, s>>>((const uint16_t *)logits, n_tokens, n_experts, n_groups,
+                                                    topk_groups, topk, score_fun, (const uint16_t *)bias,
+                                                    renormalize, ids, (uint16_t *)weights);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+extern "C" int mlk_moe_align_tokens(const int32_t *topk_ids, int n_pairs, int n_experts, int block,
+                                    const int32_t *experts_map, int32_t *sorted_token_ids, int32_t *cumsum_buffer,
+                                    int32_t *padded_num_blocks, int32_t *experts_ids, void *stream) {
+    MLK_REQUIRE(block == 16, "align: the block size must be 16");
+    MLK_REQUIRE(n_experts >= 1 && n_experts <= kMaxExperts, "align: 1..256 experts");
+    MLK_REQUIRE(n_pairs >= 0, "align: negative pair count");
+    MLK_REQUIRE(sorted_token_ids && cumsum_buffer && padded_num_blocks && experts_ids, "align: null pointer");
+    MLK_REQUIRE(n_pairs == 0 || topk_ids, "align: null pointer");
+    const int max_blocks = (n_pairs + n_experts * 15 + 15) / 16;
+    moe_align_kernel<<<1, 1024, 0, (hipStream_t)stream>>>(topk_ids, n_pairs, n_experts, experts_map, sorted_token_ids,
+                                                          cumsum_buffer, padded_num_blocks, experts_ids, max_blocks,
+                                                          nullptr, nullptr, 1);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+extern "C" size_t mlk_moe_workspace_bytes(int n_tokens, int n_experts, int topk, int hidden, int inter) {
+    (void)hidden;
+    int tc = n_tokens < kMoeChunk ? n_tokens : kMoeChunk;
+    return carve(nullptr, tc, n_experts, topk, inter, nullptr);
+}
+
+extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const void *x, int n_tokens, int n_experts,
+                                         int topk, int hidden, int inter, int w_kind, int x_kind,
+                                         const int32_t *topk_ids, const void *topk_weights,
+                                         const int32_t *experts_map, const float *w1_scale, const float *w2_scale,
+                                         void *y, void *workspace, size_t workspace_bytes, void *stream) {
+    MLK_REQUIRE(x_kind == MLK_F16 || x_kind == MLK_BF16, "moe: activations must be fp16 or bf16");
+    MLK_REQUIRE(n_tokens >= 0, "moe: negative token count");
+    MLK_REQUIRE(n_experts >= 1 && n_experts <= kMaxExperts, "moe: 1..256 experts");
+    MLK_REQUIRE(topk >= 1 && topk <= kMaxTopK, "moe: topk must be in 1..32");
+    MLK_REQUIRE(hidden > 0 && inter > 0 && hidden % 128 == 0 && inter % 128 == 0,
+                "moe: hidden and intermediate sizes must be multiples of 128");
+    const bool fp8 = w_kind == MLK_FP8_E4M3;
+    if (fp8) MLK_REQUIRE(x_kind == MLK_BF16, "moe: soft-FP8 weights need bf16 activations");
+    else MLK_REQUIRE(w_kind == x_kind, "moe: weights and activations must have the same 16-bit type");
+    if (n_tokens == 0) return MLK_OK;
+    MLK_REQUIRE(w1 && w2 && x && y && topk_ids && topk_weights && workspace, "moe: null pointer");
+    MLK_REQUIRE(workspace_bytes >= mlk_moe_workspace_bytes(n_tokens, n_experts, topk, hidden, inter),
+                "moe: workspace too small");
+    hipStream_t s = (hipStream_t)stream;
+
+    for (int t0 = 0; t0 < n_tokens; t0 += kMoeChunk) {
+        const int tc = n_tokens - t0 < kMoeChunk ? n_tokens - t0 : kMoeChunk;
+        const int n_pairs = tc * topk;
+        const int cb = (tc + 15) / 16 < 4 ? (tc + 15) / 16 : 4;   // an expert sees at most tc tokens
+        MoeWorkspace ws;
+        carve((uint8_t *)workspace, tc, n_experts, topk, inter, &ws);
+        const int max_padded = n_pairs + n_experts * 15;
+        const int max_blocks = (max_padded + 15) / 16;
+        const int active = n_experts < n_pairs ? n_experts : n_pairs;
+        const int max_tasks = active + n_pairs / (16 * cb);
+        moe_align_kernel<<<1, 1024, 0, s>>>(topk_ids + (size_t)t0 * topk, n_pairs, n_experts, experts_map, ws.sorted,
+                                            ws.cumsum, ws.padded, ws.experts_ids, max_blocks, ws.tasks, ws.n_tasks,
+                                            cb);
+        MLK_LAUNCH_CHECK();
+        MoeArgs a;
+        a.W1 = (const uint8_t *)w1;
+        a.W2 = (const uint8_t *)w2;
+        a.S1 = w1_scale;
+        a.S2 = w2_scale;
+        a.X = (const uint16_t *)x + (size_t)t0 * hidden;
+        a.Y = (uint16_t *)y + (size_t)t0 * hidden;
+        a.Hbuf = ws.hbuf;
+        a.wts = (const uint16_t *)topk_weights + (size_t)t0 * topk;
+        a.sorted = ws.sorted;
+        a.tasks = ws.tasks;
+        a.n_tasks = ws.n_tasks;
+        a.T = tc;
+        a.K = topk;
+        a.H = hidden;
+        a.I = inter;
+        a.SB = max_blocks;
+        a.n_pairs = n_pairs;
+        a.WK = 1;
+        int rc;
+        if (fp8) rc = launch_moe_cb<BF16, true>(a, cb, max_tasks, s);
+        else if (x_kind == MLK_F16) rc = launch_moe_cb<F16, false>(a, cb, max_tasks, s);
+        else rc = launch_moe_cb<BF16, false>(a, cb, max_tasks, s);
+        if (rc != MLK_OK) return rc;
+    }
+    return MLK_OK;
 }

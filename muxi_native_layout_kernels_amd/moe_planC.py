@@ -1,0 +1,118 @@
+"""Fused MoE layer entry point; same signature and defaults as the reference's
+`muxi_moe_planC.fused_moe` (muxi_layout_kernels/muxi_moe_planC.py:6-149).
+
+Three library calls per layer: router (scores, grouped selection, top-K and the
+optional renormalisation in one kernel), then alignment + grouped gate/up GeMM +
+grouped down GeMM inside `mlk_fused_experts_compute`.  Apart from the output
+nothing is allocated after the first call of a given shape: routing tables and
+the kernel workspace are cached per device.
+"""
+import threading
+from typing import List, Optional
+
+import torch
+
+from . import ops
+
+_cache_lock = threading.Lock()
+_route_cache = {}
+
+
+def _routing_buffers(n_tokens, topk, dtype, device):
+    key = (n_tokens, topk, dtype, device.type, device.index)
+    with _cache_lock:
+        hit = _route_cache.get(key)
+        if hit is None:
+            if len(_route_cache) > 64:
+                _route_cache.clear()
+            hit = (torch.empty(n_tokens, topk, dtype=torch.int32, device=device),
+                   torch.empty(n_tokens, topk, dtype=dtype, device=device))
+            _route_cache[key] = hit
+        return hit
+
+
+def fused_moe(
+    hidden_states: torch.Tensor,  # [batch_size, hidden_size]
+    w1: torch.Tensor,             # [E, 2I, H] per-expert layout-A slabs (or [E, 2I/16, H/8, 16, 8])
+    w2: torch.Tensor,             # [E, H, I]
+    gating_output: torch.Tensor,  # [batch_size, num_experts]
+    topk: int,
+    renormalize: bool,
+    use_grouped_topk: bool = False,
+    num_expert_group: Optional[int] = None,
+    topk_group: Optional[int] = None,
+    w1_scale: Optional[torch.Tensor] = None,
+    w2_scale: Optional[torch.Tensor] = None,
+    block_shape: Optional[List[int]] = None,
+    gating_bias: Optional[torch.Tensor] = None,
+    score_func: str = "softmax",
+    soft_fp8: bool = False,
+    APerWarp: int = 2,
+    splitK: int = 3,
+    tile_m_2: int = 128,
+    tile_n_2: int = 16,
+    tile_k_2: int = 128,
+    block_dim_x_gemm: int = 256,
+    experts_map: Optional[torch.Tensor] = None,
+) -> torch.Tensor:
+    """The MetaX tile parameters (APerWarp .. block_dim_x_gemm) are accepted and ignored."""
+    assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
+    if num_expert_group is None:
+        num_expert_group = 1
+    if topk_group is None:
+        topk_group = 1
+    if not use_grouped_topk and num_expert_group != 1:
+        raise ValueError("When use_grouped_topk is False, num_expert_group must be 1.")
+    if score_func == "softmax":
+        score_fun = 0
+    elif score_func == "sigmoid":
+        score_fun = 1
+    else:
+        raise ValueError("Unsupported scoring function")
+
+    shape = hidden_states.size()
+    B, H = hidden_states.shape
+    ops._check(hidden_states.is_cuda and hidden_states.is_contiguous(), "hidden_states must be a contiguous CUDA tensor")
+    ops._check(hidden_states.dtype in ops._KIND, "hidden_states must be fp16 or bf16")
+    ops._check(gating_output.dtype == hidden_states.dtype, "gating_output must have the activation dtype")
+    topk_ids, topk_weights = _routing_buffers(B, topk, hidden_states.dtype, hidden_states.device)
+    ops.fused_routing_gate(gating_output, score_fun, B, H, num_expert_group, topk_group, topk_ids, topk_weights, topk,
+                           gating_bias, renormalize=bool(renormalize))
+
+    if w1.dim() == 5:
+        e1, m1, k1 = w1.shape[0], w1.shape[1] * 16, w1.shape[2] * 8
+        e2, m2, k2 = w2.shape[0], w2.shape[1] * 16, w2.shape[2] * 8
+    else:
+        e1, m1, k1 = w1.shape
+        e2, m2, k2 = w2.shape
+    assert e1 == e2
+    assert k1 == m2
+    ops._check(k1 == H and m1 == 2 * k2, "w1 must be [E, 2I, H] and w2 [E, H, I]")
+    ops._check(w1.is_cuda and w2.is_cuda and w1.is_contiguous() and w2.is_contiguous(),
+               "expert weights must be contiguous CUDA tensors")
+    ops._check(H % 128 == 0 and k2 % 128 == 0, "hidden and intermediate sizes must be multiples of 128")
+
+    if soft_fp8:
+        assert w1_scale is not None and w2_scale is not None
+        ops._check(w1.element_size() == 1 and w2.element_size() == 1, "soft_fp8 needs one e4m3 byte per weight")
+        ops._check(hidden_states.dtype == torch.bfloat16, "Weight date type and activation date type mismatch")
+        ops._check(block_shape is not None and list(block_shape) == [128, 128],
+                   "block_shape must be (128, 128) for float8_e4m3fn.")
+        ops._check(w1_scale.dtype == torch.float32 and w2_scale.dtype == torch.float32, "scales must be float32.")
+        ops._check(tuple(w1_scale.shape) == (e1, m1 // 128, k1 // 128) and w1_scale.is_contiguous(),
+                   "w1_scale must be [E, 2I/128, H/128]")
+        ops._check(tuple(w2_scale.shape) == (e2, m2 // 128, k2 // 128) and w2_scale.is_contiguous(),
+                   "w2_scale must be [E, H/128, I/128]")
+        w_kind = ops._FP8_KIND
+    else:
+        ops._check(w1.dtype == hidden_states.dtype and w2.dtype == hidden_states.dtype,
+                   "Weight date type and activation date type mismatch")
+        w_kind = ops._KIND[w1.dtype]
+        w1_scale = w2_scale = None
+    if experts_map is not None and experts_map.dtype != torch.int:
+        experts_map = experts_map.to(torch.int)
+
+    y = torch.empty_like(hidden_states)
+    ops.experts_compute_raw(w1, w2, hidden_states, B, e1, topk, H, k2, w_kind, topk_ids, topk_weights, experts_map,
+                            w1_scale, w2_scale, y)
+    return y.view(shape)

@@ -502,17 +502,25 @@ def fused_experts_compute(experts_weights_matrix1, experts_weights_matrix2, acti
         _check(tuple(w2_scale.shape) == (e2, m2 // 128, k2 // 128) and w2_scale.is_contiguous(),
                "w2_scale must be [E, H/128, I/128]")
     experts_map = opts["experts_map"]
+    if experts_map is not None:
+        _check(experts_map.dtype == torch.int32 and experts_map.is_cuda, "experts_map must be an int32 CUDA tensor")
+    # the reference fills the caller's alignment buffers as a side effect of this call
     batched_routed_activation_indexed_to_expert_block_indexed(T, e1, K, 16, topk_ids, sorted_token_ids, cumsum_buffer,
                                                               padded_num_experts, experts_ids, experts_map)
-    lib = _lib.load()
-    ws_bytes = lib.mlk_moe_workspace_bytes(T, e1, K, hidden, inter)
-    ws = _moe_workspace(x.device, ws_bytes)
-    _lib.check(lib.mlk_fused_experts_compute(_ptr(w1), _ptr(w2), _ptr(x), T, e1, K, hidden, inter, w_kind,
-                                             _KIND[x.dtype], _ptr(actived_experts_weights), _ptr(sorted_token_ids),
-                                             _ptr(padded_num_experts), _ptr(experts_ids), _ptr(w1_scale),
-                                             _ptr(w2_scale), _ptr(y), _ptr(ws), ws.numel(), _stream()),
-               "fused_experts_compute")
+    experts_compute_raw(w1, w2, x, T, e1, K, hidden, inter, w_kind, topk_ids, actived_experts_weights, experts_map,
+                        w1_scale, w2_scale, y)
     return None
+
+
+def experts_compute_raw(w1, w2, x, T, E, K, hidden, inter, w_kind, topk_ids, topk_weights, experts_map, w1_scale,
+                        w2_scale, y):
+    """Thin call of the C entry point (alignment + both grouped GeMMs + weighted sum); no checks."""
+    lib = _lib.load()
+    ws = _moe_workspace(x.device, lib.mlk_moe_workspace_bytes(T, E, K, hidden, inter))
+    _lib.check(lib.mlk_fused_experts_compute(_ptr(w1), _ptr(w2), _ptr(x), T, E, K, hidden, inter, w_kind,
+                                             _KIND[x.dtype], _ptr(topk_ids), _ptr(topk_weights), _ptr(experts_map),
+                                             _ptr(w1_scale), _ptr(w2_scale), _ptr(y), _ptr(ws), ws.numel(),
+                                             _stream()), "fused_experts_compute")
 
 
 # ------------------------------------------------- names outside the hot path
@@ -539,5 +547,5 @@ __all__ = [
     "gemm_layoutA_soft_fp8_wapper", "gemm_layoutAB_ContinuousC_wapper", "gemv_layoutA_wapper", "fp8_weight_repack",
     "routing_gate", "experts_compute", "fused_routing_gate",
     "batched_routed_activation_indexed_to_expert_block_indexed", "fused_experts_compute",
-    "pack_layout_a", "unpack_layout_a",
+    "pack_layout_a", "unpack_layout_a", "experts_compute_raw",
 ]

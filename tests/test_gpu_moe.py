@@ -1,0 +1,258 @@
+"""GPU parity: router, alignment and the fused MoE layer against the oracle, through the C ABI.
+Indices and the permutation are bit-exact; layer outputs within rtol = atol = 1e-2 of the float64
+statement on the un-packed weights."""
+import json
+import os
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import router as orouter, align as oalign, moe as omoe, layouts
+from helpers import randn, pack_a, fp8_codes, assert_close
+
+pytestmark = pytest.mark.gpu
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+RTOL = ATOL = 1e-2
+
+
+def _route_gpu(mlk, logits, score_fun, n_groups, topk_groups, topk, bias=None, renorm=False):
+    T = logits.shape[0]
+    ids = torch.empty(T, topk, dtype=torch.int32, device="cuda")
+    w = torch.empty(T, topk, dtype=logits.dtype, device="cuda")
+    mlk.fused_routing_gate(logits.cuda(), score_fun, T, 4096, n_groups, topk_groups, ids, w, topk,
+                           None if bias is None else bias.cuda(), renormalize=renorm)
+    return ids.cpu(), w.cpu()
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("score_fun", [0, 1])
+@pytest.mark.parametrize("T,E,K", [(1, 8, 2), (16, 8, 2), (256, 8, 2), (77, 64, 6), (33, 256, 8), (5, 16, 16)])
+def test_router_plain(mlk, dtype, score_fun, T, E, K):
+    logits = randn((T, E), dtype, 1.0, 2025 + T)
+    ids, w = _route_gpu(mlk, logits, score_fun, 1, 1, K)
+    ids_o, w_o = orouter.route(logits, score_fun, 1, 1, K)
+    assert torch.equal(ids, ids_o)
+    assert torch.equal(w.view(torch.int16), w_o.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("score_fun", [0, 1])
+@pytest.mark.parametrize("with_bias", [False, True])
+def test_router_grouped_deepseek_configuration(mlk, dtype, score_fun, with_bias):
+    T, E = 64, 256
+    logits = randn((T, E), dtype, 1.0, 31)
+    bias = randn((E,), dtype, 0.05, 32).abs() if with_bias else None
+    ids, w = _route_gpu(mlk, logits, score_fun, 8, 4, 8, bias)
+    ids_o, w_o = orouter.route(logits, score_fun, 8, 4, 8, bias)
+    assert torch.equal(ids, ids_o)
+    assert torch.equal(w.view(torch.int16), w_o.view(torch.int16))
+
+
+def test_router_special_cases_and_renorm(mlk):
+    eq = torch.zeros((3, 16), dtype=torch.bfloat16)
+    ids, w = _route_gpu(mlk, eq, 0, 1, 1, 4)
+    assert ids.tolist() == [[0, 1, 2, 3]] * 3
+    logits = randn((128, 8), torch.bfloat16, 1.0, 5)
+    ids, w = _route_gpu(mlk, logits, 0, 1, 1, 2, renorm=True)
+    ids_o, w_o = orouter.route(logits, 0, 1, 1, 2)
+    assert torch.equal(ids, ids_o)
+    assert torch.equal(w.view(torch.int16), orouter.renormalize(w_o).view(torch.int16))
+    # the same division done by torch on the GPU, as the reference's caller does it
+    _, w_plain = _route_gpu(mlk, logits, 0, 1, 1, 2)
+    wp = w_plain.cuda()
+    assert torch.equal(w.cuda(), wp / wp.sum(dim=-1, keepdim=True))
+
+
+def _align_gpu(mlk, ids, E, K, emap=None):
+    T = ids.shape[0]
+    n = T * K
+    padded = n + E * 15
+    dev = "cuda"
+    s = torch.empty(padded, dtype=torch.int32, device=dev)
+    cs = torch.empty(E + 1, dtype=torch.int32, device=dev)
+    pn = torch.empty(1, dtype=torch.int32, device=dev)
+    ei = torch.empty((padded + 15) // 16, dtype=torch.int32, device=dev)
+    mlk.batched_routed_activation_indexed_to_expert_block_indexed(
+        T, E, K, 16, ids.to(torch.int32).cuda(), s, cs, pn, ei,
+        None if emap is None else torch.as_tensor(emap, dtype=torch.int32).cuda())
+    return s.cpu().numpy(), cs.cpu().numpy(), int(pn.item()), ei.cpu().numpy()
+
+
+def _compare_align(got, want):
+    s, cs, pn, ei = got
+    assert np.array_equal(s, want["sorted_token_ids"])
+    assert np.array_equal(cs[:-1], want["cursors"][:-1]) and cs[-1] == want["cumsum"][-1]
+    assert pn == want["padded_num_blocks"]
+    assert np.array_equal(ei, want["experts_ids"])
+
+
+def test_align_reference_example(mlk):
+    ex = json.load(open(os.path.join(GOLD, "align_example_topk_ids.json")))
+    ids = torch.tensor(ex["topk_ids"]).reshape(ex["tokens"], ex["topk"])
+    _compare_align(_align_gpu(mlk, ids, ex["num_experts"], ex["topk"]),
+                   oalign.align_tokens(ex["topk_ids"], ex["num_experts"]))
+
+
+@pytest.mark.parametrize("T,K,E", [(1, 2, 8), (16, 2, 8), (64, 2, 8), (256, 2, 8), (33, 8, 256), (2048, 8, 256),
+                                   (1000, 6, 64), (3, 1, 5)])
+def test_align_random(mlk, T, K, E):
+    rng = np.random.default_rng(T * 31 + K)
+    ids = torch.from_numpy(np.stack([rng.choice(E, size=K, replace=False) for _ in range(T)]))
+    _compare_align(_align_gpu(mlk, ids, E, K), oalign.align_tokens(ids.numpy(), E))
+
+
+def test_align_expert_map(mlk):
+    rng = np.random.default_rng(1)
+    ids = torch.from_numpy(np.stack([rng.choice(16, size=4, replace=False) for _ in range(200)]))
+    emap = np.array([e // 2 if e % 2 == 0 else -1 for e in range(16)])
+    _compare_align(_align_gpu(mlk, ids, 8, 4, emap), oalign.align_tokens(ids.numpy(), 8, experts_map=emap))
+
+
+def _pack_experts(w):
+    return torch.stack([pack_a(w[e]) for e in range(w.shape[0])]).reshape(w.shape)
+
+
+def _moe_case(mlk, T, E, K, H, I, dtype, seed, score="softmax", fp8=False, groups=None, bias=None, emap=None):
+    from muxi_native_layout_kernels_amd.moe_planC import fused_moe
+    x = randn((T, H), dtype, 1.0, seed)
+    logits = randn((T, E), dtype, 1.0, seed + 1)
+    kw = {}
+    if fp8:
+        c1 = fp8_codes((E, 2 * I, H), seed + 2, std=1.0)
+        c2 = fp8_codes((E, H, I), seed + 3, std=1.0)
+        g = torch.Generator().manual_seed(seed + 4)
+        s1 = (torch.rand((E, 2 * I // 128, H // 128), generator=g) * 0.03 + 0.005).float()
+        s2 = (torch.rand((E, H // 128, I // 128), generator=g) * 0.03 + 0.005).float()
+        w1u = omoe.dequant_experts(c1.numpy(), s1.numpy())
+        w2u = omoe.dequant_experts(c2.numpy(), s2.numpy())
+        w1p, w2p = _pack_experts(c1), _pack_experts(c2)
+        kw = dict(w1_scale=s1.cuda(), w2_scale=s2.cuda(), block_shape=[128, 128], soft_fp8=True)
+    else:
+        w1u = randn((E, 2 * I, H), dtype, 0.02, seed + 2)
+        w2u = randn((E, H, I), dtype, 0.02, seed + 3)
+        w1p, w2p = _pack_experts(w1u), _pack_experts(w2u)
+    n_groups, tk_groups = groups if groups else (1, 1)
+    y = fused_moe(x.cuda(), w1p.cuda(), w2p.cuda(), logits.cuda(), K, True, use_grouped_topk=groups is not None,
+                  num_expert_group=n_groups, topk_group=tk_groups, gating_bias=None if bias is None else bias.cuda(),
+                  score_func=score, experts_map=None if emap is None else torch.as_tensor(emap).cuda(), **kw)
+    assert y.shape == x.shape and y.dtype == dtype
+    ids, wts = orouter.route(logits, 0 if score == "softmax" else 1, n_groups, tk_groups, K, bias)
+    wts = orouter.renormalize(wts)
+    want = omoe.moe_expected(x, w1u, w2u, ids, wts, round_h_to=dtype, expert_map=emap)
+    assert_close(y, want, RTOL, ATOL, "fused_moe T=%d" % T)
+    return y
+
+
+@pytest.mark.parametrize("T", [1, 2, 16, 17, 64, 100, 256, 300])
+def test_fused_moe_small_shape(mlk, T):
+    _moe_case(mlk, T, 8, 2, 256, 384, torch.bfloat16, 100 + T)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_fused_moe_dtypes_and_determinism(mlk, dtype):
+    y1 = _moe_case(mlk, 40, 8, 2, 512, 256, dtype, 7)
+    y2 = _moe_case(mlk, 40, 8, 2, 512, 256, dtype, 7)
+    assert torch.equal(y1, y2)
+
+
+@pytest.mark.parametrize("T", [1, 16, 70])
+def test_fused_moe_soft_fp8(mlk, T):
+    _moe_case(mlk, T, 8, 2, 256, 384, torch.bfloat16, 300 + T, fp8=True)
+
+
+def test_fused_moe_grouped_sigmoid_bias(mlk):
+    E = 64
+    bias = randn((E,), torch.bfloat16, 0.05, 9).abs()
+    _moe_case(mlk, 24, E, 8, 256, 128, torch.bfloat16, 500, score="sigmoid", groups=(8, 4), bias=bias)
+
+
+def test_fused_moe_expert_map(mlk):
+    emap = np.array([0, -1, 1, -1, 2, -1, 3, -1], dtype=np.int32)
+    # local experts 0..3 hold the weights of global experts 0, 2, 4, 6
+    from muxi_native_layout_kernels_amd.moe_planC import fused_moe
+    T, E, K, H, I = 32, 8, 2, 256, 256
+    dtype = torch.bfloat16
+    x = randn((T, H), dtype, 1.0, 1)
+    logits = randn((T, E), dtype, 1.0, 2)
+    w1 = randn((4, 2 * I, H), dtype, 0.02, 3)
+    w2 = randn((4, H, I), dtype, 0.02, 4)
+    y = fused_moe(x.cuda(), _pack_experts(w1).cuda(), _pack_experts(w2).cuda(), logits.cuda(), K, True,
+                  experts_map=torch.as_tensor(emap).cuda())
+    ids, wts = orouter.route(logits, 0, 1, 1, K)
+    want = omoe.moe_expected(x, w1, w2, ids, orouter.renormalize(wts), round_h_to=dtype, expert_map=emap)
+    assert_close(y, want, RTOL, ATOL, "expert map")
+
+
+def test_fused_moe_matches_torch_path_on_gpu(mlk):
+    """The reference's own test recipe: compare with the pure-torch MoE run on the GPU in the same dtype,
+    atol 0.1 / rtol 0.05 (benchmark_and_test/test_muxi_moe.py:111)."""
+    from muxi_native_layout_kernels_amd.moe_planC import fused_moe
+    from muxi_native_layout_kernels_amd import utils
+    T, E, K, H, I = 48, 8, 2, 512, 768
+    dtype = torch.bfloat16
+    x = (torch.rand((T, H), generator=torch.Generator().manual_seed(1)) / 100).to(dtype)
+    logits = randn((T, E), dtype, 1.0, 2)
+    w1 = (torch.rand((E, 2 * I, H), generator=torch.Generator().manual_seed(3)) / 10).to(dtype)
+    w2 = (torch.rand((E, H, I), generator=torch.Generator().manual_seed(4)) / 10).to(dtype)
+    y = fused_moe(x.cuda(), _pack_experts(w1).cuda(), _pack_experts(w2).cuda(), logits.cuda(), K, True)
+    ref = utils.fused_moe(x.cuda(), w1.cuda(), w2.cuda(), logits.cuda(), K, num_expert_group=1, topk_group=1,
+                          global_num_experts=E, renormalize=True)
+    torch.testing.assert_close(y, ref, atol=0.1, rtol=0.05)
+
+
+def test_low_level_fused_experts_compute_signature(mlk):
+    """Call sequence of the reference's Python entry (muxi_moe_planC.py:44-146) on the low-level ops."""
+    T, E, K, H, I = 20, 8, 2, 256, 256
+    dtype = torch.float16
+    x = randn((T, H), dtype, 1.0, 1).cuda()
+    logits = randn((T, E), dtype, 1.0, 2).cuda()
+    w1u = randn((E, 2 * I, H), dtype, 0.02, 3)
+    w2u = randn((E, H, I), dtype, 0.02, 4)
+    w1, w2 = _pack_experts(w1u).cuda(), _pack_experts(w2u).cuda()
+    ids = torch.empty(T, K, dtype=torch.int32, device="cuda")
+    wts = torch.empty(T, K, dtype=dtype, device="cuda")
+    mlk.fused_routing_gate(logits, 0, T, H, 1, 1, ids, wts, K, None)
+    wts = wts / wts.sum(dim=-1, keepdim=True)
+    padded = K * T + E * 15
+    sorted_ids = torch.full((padded,), T * K, dtype=torch.int32, device="cuda")
+    cumsum = torch.empty(E + 1, dtype=torch.int32, device="cuda")
+    pn = torch.empty(1, dtype=torch.int32, device="cuda")
+    eids = torch.empty((padded + 15) // 16, dtype=torch.int32, device="cuda")
+    C = torch.zeros(K * 2 * I * T, dtype=dtype, device="cuda")
+    y = torch.zeros_like(x)
+    mlk.fused_experts_compute(w1, w2, x, T, E, K, ids, wts, sorted_ids, cumsum, pn, eids, C, y, APerWarp=2, splitK=3,
+                              tile_m_2=128, tile_n_2=16, tile_k_2=128, block_dim_x_gemm=256, experts_map=None)
+    want = omoe.moe_expected(x.cpu(), w1u, w2u, ids.cpu(), wts.cpu(), round_h_to=dtype)
+    assert_close(y, want, RTOL, ATOL, "low-level")
+    assert int(pn.item()) == oalign.align_tokens(ids.cpu().numpy(), E)["padded_num_blocks"]
+
+
+@pytest.mark.parametrize("T", [1, 16])
+def test_fused_moe_mixtral_shape(mlk, T):
+    """E=8, top-2, H=4096, I=14336 at full size; the oracle only evaluates the selected experts."""
+    from muxi_native_layout_kernels_amd.moe_planC import fused_moe
+    E, K, H, I = 8, 2, 4096, 14336
+    dtype = torch.bfloat16
+    x = randn((T, H), dtype, 1.0, 2025)
+    logits = randn((T, E), dtype, 1.0, 2026)
+    g = torch.Generator(device="cuda").manual_seed(2027)
+    w1u = (torch.randn((E, 2 * I, H), generator=g, device="cuda") * 0.02).to(dtype)
+    w2u = (torch.randn((E, H, I), generator=g, device="cuda") * 0.02).to(dtype)
+    w1p = mlk.pack_layout_a(w1u).view(E, 2 * I, H)
+    w2p = mlk.pack_layout_a(w2u).view(E, H, I)
+    y = fused_moe(x.cuda(), w1p, w2p, logits.cuda(), K, True)
+    ids, wts = orouter.route(logits, 0, 1, 1, K)
+    wts = orouter.renormalize(wts)
+    tok = list(range(T)) if T <= 4 else [0, T // 2, T - 1]    # bound the float64 work on the host
+    w1c, w2c = {}, {}
+    for t in tok:
+        for e in ids[t].tolist():
+            if e not in w1c:
+                w1c[e], w2c[e] = w1u[e].cpu(), w2u[e].cpu()
+    class Lazy:
+        def __init__(self, d, shape): self.d, self.shape = d, shape
+        def __getitem__(self, e): return self.d[e]
+    want = omoe.moe_expected(x[tok], Lazy(w1c, (E, 2 * I, H)), Lazy(w2c, (E, H, I)), ids[tok], wts[tok],
+                             round_h_to=dtype)
+    assert_close(y[tok], want, RTOL, ATOL, "mixtral T=%d" % T)

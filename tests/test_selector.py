@@ -1,0 +1,75 @@
+"""CPU: csv dispatch tables - parse rules, fallbacks, guard rails, shipped tables."""
+import os
+
+import pytest
+
+from oracle import selector as osel
+from muxi_native_layout_kernels_amd import arg_selector
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def test_excerpt_known_answers_oracle_and_product_agree():
+    text = open(os.path.join(GOLD, "gemv_bf16_excerpt.csv")).read()
+    want = osel.parse_table(text, 2)
+    got = arg_selector.parse_table_text(text, 2)
+    assert got == want
+    # three rows share the key (4096, 4096); the last one wins (reference table line 45)
+    assert got[(4096, 4096)] == (256, 1, 1, 3)
+    # the 5-cell row is skipped
+    assert (1024, 4096) not in got
+    assert got[(19008, 5120)] == (256, 1, 1, 8)
+
+
+def test_known_answer_rows_parse():
+    rows = [l for l in open(os.path.join(GOLD, "selector_rows.csv")).read().splitlines() if not l.startswith("#")]
+    for line in rows:
+        fname, lineno, row = line.split(",", 2)
+        cells = [int(c) for c in row.strip('"').split(",")]
+        nkey = 2 if "gemv" in fname else 3
+        table = osel.parse_table("header\n" + ",".join(map(str, cells)), nkey)
+        assert table[tuple(cells[:nkey])] == tuple(cells[nkey:])
+
+
+def test_fallbacks_and_guards_oracle():
+    assert osel.lookup({}, (1, 2, 3), osel.GEMM_FALLBACK) == (1, 1, 1, 1)
+    assert osel.lookup({}, (1, 2), osel.GEMV_FALLBACK) == (256, 1, 1, 1)
+    assert osel.gemv_guard((256, 1, 3, 1), 4096, 4096) == (256, 1, 1, 1)   # 256 row groups % 3 != 0
+    assert osel.gemv_guard((256, 2, 16, 0), 4096, 16384) == (256, 1, 1, 1)  # kernel 2 needs k <= 8192
+    assert osel.gemv_guard((128, 1, 2, 1), 4096, 4096) == (128, 1, 2, 1)
+
+
+def test_product_selector_miss_is_memoised_and_warns_once(capsys, tmp_path, monkeypatch):
+    sel = arg_selector._Selector("does_not_exist.csv", 3, arg_selector.GEMM_FALLBACK, "test GEMM")
+    a = sel.get_args((128, 16, 128))
+    b = sel.get_args((128, 16, 128))
+    err = capsys.readouterr().err
+    assert a == b == (1, 1, 1, 1)
+    assert err.count("No matching arguments") == 1
+    assert "Error opening file" in err
+
+
+def test_product_selector_reads_table(tmp_path):
+    p = tmp_path / "t.csv"
+    p.write_text("m,n,k,kernelId,kernelParam1,kernelParam2,kernelParam3\n128,16,256,1,2,4,1\nbad,row\n128,16,256,1,4,8,1\n")
+    sel = arg_selector._Selector(str(p), 3, arg_selector.GEMM_FALLBACK, "tmp")
+    sel.path = lambda: str(p)
+    assert sel.get_args((128, 16, 256)) == (1, 4, 8, 1)
+
+
+def test_gemv_guard_product():
+    assert arg_selector.gemv_guard((512, 1, 2, 4), 4096, 4096) == (512, 1, 2, 4)
+    assert arg_selector.gemv_guard((512, 1, 3, 4), 4096, 4096) == (256, 1, 1, 4)
+    assert arg_selector.gemv_guard((100, 1, 1, 4), 4096, 4096) == (256, 1, 1, 4)
+
+
+@pytest.mark.parametrize("name", ["layout_gemm", "continuous_gemm", "layoutA_gemm", "layoutA_soft_fp8_gemm",
+                                  "gemv_fp16", "gemv_bf16", "gemv_soft_fp8"])
+def test_shipped_tables_parse(name):
+    sel = arg_selector.selector(name)
+    assert os.path.exists(sel.path()), "every selector ships its table"
+    table = sel.table()
+    text = open(sel.path()).read()
+    assert table == osel.parse_table(text, sel.key_cells)
+    for key, val in table.items():
+        assert len(key) == sel.key_cells and len(val) == 4
