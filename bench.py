@@ -1,0 +1,285 @@
+#!/usr/bin/env python3
+"""Benchmark of the native-layout hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+
+Prints ONE JSON line.  The headline workload is the fp16 narrow GeMM of the
+second benchmark configuration (`gemm_layoutA`, weights 11008 x 4096 in
+layout-A, 16 tokens); one step is one call.  Inputs are synthetic, seeded and
+resident in HBM before the timed region.  Every call of a timed region reads a
+different weight copy (enough copies to exceed the 256 MiB Infinity Cache), so
+the bandwidth is HBM bandwidth.  The K timed calls are replayed from one HIP
+graph, bracketed by HIP events on the stream that runs them.
+
+`per_config` in the same line holds the other configurations (bf16 / soft-FP8
+GeMV, the M sweep, the native-layout chain and the fused MoE layer) with
+microseconds per call, achieved GB/s of algorithmic bytes and the fraction of
+the 8 TB/s HBM peak.  `cpu_baseline` is the reference's CPU-runnable path (a
+library linear on the un-packed weights in the same dtype) timed on the host
+cores on a bounded sample.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+MALL_BYTES = 256 << 20
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=50)
+    ap.add_argument("--quick", action="store_true", help="headline workload only")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain copy kernel of known size (256 MiB in, 256 MiB out) so that "
+                         "hardware byte counters can be scaled against it")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    import muxi_native_layout_kernels_amd as mlk
+    from muxi_native_layout_kernels_amd import _lib, arg_selector
+    from muxi_native_layout_kernels_amd.moe_planC import fused_moe
+    lib = _lib.load()
+    dev = torch.device("cuda:0")
+    torch.cuda.set_device(dev)
+    gen = torch.Generator(device=dev).manual_seed(2025)
+    DT = {0: torch.float16, 1: torch.bfloat16}
+
+    def copies_for(nbytes):
+        return int(max(2, min(24, (3 * MALL_BYTES + nbytes - 1) // nbytes)))
+
+    def weights(n, k, kind, count):
+        """`count` independent weight tensors, already in layout-A (values are i.i.d., so drawing
+        them directly in packed order is the same distribution as packing a drawn matrix)."""
+        out = []
+        for _ in range(count):
+            if kind == 2:
+                w = (torch.randn((n // 16, k // 8, 16, 8), generator=gen, device=dev) * 16).clamp_(-448, 448)
+                out.append(w.to(torch.float8_e4m3fn).view(torch.uint8))
+            else:
+                out.append((torch.randn((n // 16, k // 8, 16, 8), generator=gen, device=dev) * 0.02).to(DT[kind]))
+        return out
+
+    def run_graph(calls, steps, warmup):
+        """Replay `steps` calls (cycling through `calls`) from one HIP graph; returns
+        (microseconds per call from HIP events on the launching stream, wall seconds of the timed region)."""
+        stream = torch.cuda.Stream()
+        with torch.cuda.stream(stream):
+            for i in range(max(warmup, 3)):
+                calls[i % len(calls)]()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=stream):
+                for i in range(steps):
+                    calls[i % len(calls)]()
+            graph.replay()
+            torch.cuda.synchronize()
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            t0 = time.perf_counter()
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - t0
+            us = e0.elapsed_time(e1) * 1e3 / steps
+        return us, wall
+
+    def gemv_case(name, n, k, kind, steps, warmup):
+        xk = 1 if kind == 2 else kind
+        A = weights(n, k, kind, copies_for(n * k * (1 if kind == 2 else 2)))
+        x = torch.randn((1, k), generator=gen, device=dev).to(DT[xk])
+        y = torch.empty((1, n), dtype=DT[xk], device=dev)
+        scale = torch.ones(((n + 127) // 128, (k + 127) // 128), dtype=torch.float32, device=dev) if kind == 2 else None
+        sel = {0: "gemv_fp16", 1: "gemv_bf16", 2: "gemv_soft_fp8"}[kind]
+        block, kid, p1, p2 = arg_selector.gemv_guard(arg_selector.selector(sel).get_args((n, k)), n, k)
+
+        def mk(a):
+            def call():
+                st = torch.cuda.current_stream().cuda_stream
+                _lib.check(lib.mlk_gemv_layout_a(a.data_ptr(), x.data_ptr(), y.data_ptr(), 1, n, k, kind, xk, 1.0, 0,
+                                                 0 if scale is None else scale.data_ptr(), block, kid, p1, p2, st),
+                           "gemv")
+            return call
+        us, wall = run_graph([mk(a) for a in A], steps, warmup)
+        algo = n * k * (1 if kind == 2 else 2) + (scale.numel() * 4 if scale is not None else 0) + k * 2 + n * 2
+        return dict(name=name, us=us, bytes=algo, gbps=algo / us / 1e3, frac=algo / us / 1e3 / HBM_PEAK_GBPS,
+                    params=[block, kid, p1, p2], copies=len(A), wall=wall)
+
+    def gemm_case(name, n, k, kind, m, steps, warmup, native=False):
+        xk = 1 if kind == 2 else kind
+        A = weights(n, k, kind, copies_for(n * k * (1 if kind == 2 else 2)))
+        b = torch.randn((m, k), generator=gen, device=dev).to(DT[xk])
+        scale = torch.ones((n // 128, k // 128), dtype=torch.float32, device=dev) if kind == 2 else None
+        table = "layoutA_soft_fp8_gemm" if kind == 2 else ("layout_gemm" if native else "layoutA_gemm")
+        kid, p1, p2, p3 = mlk.ops._gemm_guard(arg_selector.selector(table).get_args((n, m, k)), n)
+        p3 = 1
+        if native:
+            b_in = mlk.layoutB(b)
+            c = torch.empty((n // 32, m // 16, 4, 16, 8), dtype=DT[xk], device=dev)
+            c_rm = torch.empty((m, n), dtype=DT[xk], device=dev)
+        else:
+            b_in = b
+            c = torch.empty((m, n), dtype=DT[xk], device=dev)
+
+        def mk(a):
+            def call():
+                st = torch.cuda.current_stream().cuda_stream
+                _lib.check(lib.mlk_gemm_layout_a(a.data_ptr(), b_in.data_ptr(), c.data_ptr(), m, n, k, kind, xk,
+                                                 1 if native else 0, 1 if native else 0, 1.0, 0,
+                                                 0 if scale is None else scale.data_ptr(), kid, p1, p2, p3, 0, 0, st),
+                           "gemm")
+                if native:
+                    _lib.check(lib.mlk_re_layout_c(c.data_ptr(), c_rm.data_ptr(), m, n, st), "reLayoutC")
+            return call
+        us, wall = run_graph([mk(a) for a in A], steps, warmup)
+        algo = n * k * (1 if kind == 2 else 2) + (scale.numel() * 4 if scale is not None else 0) + m * k * 2 + m * n * 2
+        if native:
+            algo += 2 * m * n * 2
+        return dict(name=name, us=us, bytes=algo, gbps=algo / us / 1e3, frac=algo / us / 1e3 / HBM_PEAK_GBPS,
+                    params=[kid, p1, p2, p3], copies=len(A), wall=wall)
+
+    moe_w = {}
+
+    def moe_case(name, T, fp8, steps, warmup):
+        E, K, H, I = 8, 2, 4096, 14336
+        key = "fp8" if fp8 else "bf16"
+        if key not in moe_w:
+            moe_w.clear()
+            torch.cuda.empty_cache()
+            if fp8:
+                w1 = (torch.randn((E, 2 * I, H), generator=gen, device=dev) * 16).clamp_(-448, 448)
+                w1 = w1.to(torch.float8_e4m3fn).view(torch.uint8)
+                w2 = (torch.randn((E, H, I), generator=gen, device=dev) * 16).clamp_(-448, 448)
+                w2 = w2.to(torch.float8_e4m3fn).view(torch.uint8)
+                s1 = torch.full((E, 2 * I // 128, H // 128), 0.02 / 16, dtype=torch.float32, device=dev)
+                s2 = torch.full((E, H // 128, I // 128), 0.02 / 16, dtype=torch.float32, device=dev)
+                moe_w[key] = (w1, w2, s1, s2)
+            else:
+                w1 = (torch.randn((E, 2 * I, H), generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+                w2 = (torch.randn((E, H, I), generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+                moe_w[key] = (w1, w2, None, None)
+        w1, w2, s1, s2 = moe_w[key]
+        x = torch.randn((T, H), generator=gen, device=dev).to(torch.bfloat16)
+        logits = torch.randn((T, E), generator=gen, device=dev).to(torch.bfloat16)
+        kw = dict(w1_scale=s1, w2_scale=s2, block_shape=[128, 128], soft_fp8=True) if fp8 else {}
+
+        def call():
+            return fused_moe(x, w1, w2, logits, K, True, **kw)
+        y = call()
+        ids = torch.topk(torch.softmax(logits.float(), dim=-1), K, dim=-1).indices
+        e_act = int(torch.unique(ids).numel())
+        us, wall = run_graph([call], steps, warmup)
+        wbytes = 1 if fp8 else 2
+        algo = e_act * 3 * I * H * wbytes + 2 * T * H * 2 + T * E * 2
+        if fp8:
+            algo += e_act * 3 * (I // 128) * (H // 128) * 4
+        del y
+        return dict(name=name, us=us, bytes=algo, gbps=algo / us / 1e3, frac=algo / us / 1e3 / HBM_PEAK_GBPS,
+                    active_experts=e_act, roofline_us=algo / HBM_PEAK_GBPS / 1e3,
+                    ratio_to_roofline=us / (algo / HBM_PEAK_GBPS / 1e3), wall=wall)
+
+    if args.calibrate_copy:
+        src = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        for _ in range(4):   # fp8_repack_kernel: one dword in, one dword out per thread
+            _lib.check(lib.mlk_fp8_weight_repack(src.data_ptr(), dst.data_ptr(), src.numel(),
+                                                 torch.cuda.current_stream().cuda_stream), "copy")
+        torch.cuda.synchronize()
+        del src, dst
+
+    # ------------------------------------------------------------ headline
+    N, K_, M = 11008, 4096, 16
+    head = gemm_case("C2 fp16 gemm_layoutA 11008x4096 M=16", N, K_, 0, M, args.steps, args.warmup)
+    per_config = []
+    if not args.quick:
+        short = max(20, min(args.steps, 100))
+        per_config.append(gemv_case("C1 bf16 gemv 4096x4096", 4096, 4096, 1, short, 10))
+        for m in (1, 8, 32, 64):
+            per_config.append(gemm_case("C2 fp16 gemm_layoutA 11008x4096 M=%d" % m, N, K_, 0, m, short, 10))
+        per_config.append(gemv_case("C2 fp16 gemv 11008x4096", N, K_, 0, short, 10))
+        per_config.append(gemv_case("C3 soft-fp8 gemv 28672x8192", 28672, 8192, 2, short, 10))
+        for m in (4, 16):
+            per_config.append(gemm_case("C3 soft-fp8 gemm_layoutA 28672x8192 M=%d" % m, 28672, 8192, 2, m, short, 10))
+        per_config.append(gemm_case("C4 bf16 gemm_layoutABC+reLayoutC 8192x8192 M=32", 8192, 8192, 1, 32, short, 10,
+                                    native=True))
+        for T in (1, 16, 64, 256):
+            per_config.append(moe_case("C5 bf16 fused_moe T=%d" % T, T, False, 20, 5))
+        for T in (1, 16):
+            per_config.append(moe_case("C5 soft-fp8 fused_moe T=%d" % T, T, True, 20, 5))
+        moe_w.clear()
+        torch.cuda.empty_cache()
+        for row in per_config:
+            row.pop("wall", None)
+            for key in ("us", "gbps", "frac", "roofline_us", "ratio_to_roofline"):
+                if key in row:
+                    row[key] = round(row[key], 4)
+
+    # -------------------------------------------------------- CPU baseline
+    cpu = None
+    if not args.no_cpu:
+        from oracle import gemm as ogemm
+        rows = 2048                                    # bounded sample: the first 2048 of 11008 weight rows
+        g = torch.Generator().manual_seed(2025)
+        w = (torch.randn((rows, K_), generator=g) * 0.02).to(torch.float16)
+        b = torch.randn((M, K_), generator=g).to(torch.float16)
+        for _ in range(2):
+            ogemm.torch_path_linear(w, b)
+        reps, t0 = 0, time.perf_counter()
+        while reps < 5 or (time.perf_counter() - t0 < 5.0 and reps < 200):
+            ogemm.torch_path_linear(w, b)
+            reps += 1
+        dt = (time.perf_counter() - t0) / reps
+        sample_bytes = rows * K_ * 2 + M * K_ * 2 + M * rows * 2
+        cpu = dict(value=round(sample_bytes / dt / 1e9, 3), unit="GB/s", cores=torch.get_num_threads(),
+                   kind="port",
+                   sample="torch linear in fp16 on the first %d of %d un-packed weight rows, M=%d, %d reps, %.3f ms each; "
+                          "host has %d logical CPUs" % (rows, N, M, reps, dt * 1e3, os.cpu_count() or 0))
+
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic = json.load(open(tpath)).get("C2 fp16 gemm_layoutA 11008x4096 M=16")
+        except (OSError, ValueError):
+            traffic = None
+
+    line = {
+        "metric": "achieved GB/s of algorithmic bytes per call (us/call and % of HBM peak alongside)",
+        "value": round(head["gbps"], 2),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(head["wall"] * 1e3 / args.steps, 6),
+        "us_per_call": round(head["us"], 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {"workload": head["name"], "weights": "fp16 N(0,0.02) in layout-A, %d rotating copies" % head["copies"],
+                   "activations": "fp16 N(0,1) row-major [16, 4096]", "launch_params": head["params"],
+                   "algorithmic_bytes": head["bytes"]},
+        "roofline": {"bound": "hbm", "achieved": round(head["gbps"], 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(head["frac"], 4), "traffic": traffic},
+        "cpu_baseline": cpu,
+        "per_config": per_config,
+    }
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()
