@@ -1,0 +1,195 @@
+"""Offline launch-parameter scan for gfx950: brute-forces the `_wapper` entry points over the
+parameter grid of each kernel, keeps the fastest configuration that passes a correctness gate and
+writes csv rows the selectors can parse.
+
+Counterpart of the reference's eight scan scripts (kernel_args_scan/gemv_kernel_args_scan.py:135-165,
+gemv_kernel_args_scan_sf8.py, gemm_kernel_args_scan_kernel_all*.py): same idea (time every
+configuration through the wapper, gate on the difference to an expected product, keep the best, emit
+`m,k,...` / `m,n,k,...` rows), with the gfx950 kernels' own parameter grids.
+
+    python -m muxi_native_layout_kernels_amd.kernel_args_scan.scan gemv_bf16 --shapes 4096x4096,28672x8192
+    python -m muxi_native_layout_kernels_amd.kernel_args_scan.scan layoutA_gemm --shapes 11008x4096 --tokens 1,8,16,32,64
+    python -m muxi_native_layout_kernels_amd.kernel_args_scan.scan all --update
+
+Tables: gemv_fp16, gemv_bf16, gemv_soft_fp8, layoutA_gemm, layoutA_soft_fp8_gemm, continuous_gemm, layout_gemm.
+`--update` appends the rows to the packaged csv (later rows win on lookup); without it they go to
+`<table>_scan_best_args.csv` in the current directory.
+
+Timing: each configuration is captured `--iters` times into one HIP graph over rotating weight
+copies that together exceed the Infinity Cache, and timed with HIP events.
+"""
+import argparse
+import sys
+
+import torch
+
+from .. import ops, arg_selector
+
+GEMV_TABLES = {"gemv_fp16": torch.float16, "gemv_bf16": torch.bfloat16, "gemv_soft_fp8": None}
+GEMM_TABLES = {"layoutA_gemm": ("rowmajor", torch.float16), "layoutA_soft_fp8_gemm": ("fp8", torch.bfloat16),
+               "continuous_gemm": ("continuous", torch.bfloat16), "layout_gemm": ("native", torch.bfloat16)}
+DEFAULT_SHAPES = {
+    "gemv_fp16": [(11008, 4096), (4096, 4096), (4096, 11008)],
+    "gemv_bf16": [(4096, 4096), (28672, 8192), (8192, 8192), (28672, 4096), (4096, 14336)],
+    "gemv_soft_fp8": [(28672, 8192), (4096, 4096), (8192, 8192)],
+    "layoutA_gemm": [(11008, 4096)],
+    "layoutA_soft_fp8_gemm": [(28672, 8192)],
+    "continuous_gemm": [(8192, 8192)],
+    "layout_gemm": [(8192, 8192)],
+}
+DEFAULT_TOKENS = {"layoutA_gemm": [1, 8, 16, 32, 64], "layoutA_soft_fp8_gemm": [1, 4, 16],
+                  "continuous_gemm": [16, 32, 64], "layout_gemm": [16, 32, 64]}
+MALL_BYTES = 256 << 20
+
+
+def _time_graph(calls, iters):
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        for c in calls[:2]:
+            c()
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(iters):
+                calls[i % len(calls)]()
+        graph.replay()
+        torch.cuda.synchronize()
+        best = float("inf")
+        for _ in range(3):
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            graph.replay()
+            e1.record()
+            torch.cuda.synchronize()
+            best = min(best, e0.elapsed_time(e1) * 1e3 / iters)
+    return best
+
+
+def _weights(n, k, dtype, fp8, count, gen):
+    out = []
+    for _ in range(count):
+        w = torch.randn((n, k), generator=gen, device="cuda")
+        if fp8:
+            out.append((w * 16).clamp_(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8))
+        else:
+            out.append((w * 0.02).to(dtype))
+    return out
+
+
+def _copies(nbytes):
+    return int(max(2, min(16, (3 * MALL_BYTES + nbytes - 1) // nbytes)))
+
+
+def _gate(got, want):
+    err = (got.float() - want).abs()
+    return bool((err <= 1e-2 + 1e-2 * want.abs()).all())
+
+
+def scan_gemv(table, shapes, iters):
+    dtype = GEMV_TABLES[table]
+    fp8 = dtype is None
+    xdt = torch.bfloat16 if fp8 else dtype
+    gen = torch.Generator(device="cuda").manual_seed(2025)
+    rows = []
+    for n, k in shapes:
+        plain = _weights(n, k, xdt, fp8, _copies(n * k * (1 if fp8 else 2)), gen)
+        packed = [ops.pack_layout_a(w) for w in plain]
+        x = torch.randn((1, k), generator=gen, device="cuda").to(xdt)
+        scale = torch.ones(((n + 127) // 128, (k + 127) // 128), dtype=torch.float32, device="cuda") if fp8 else None
+        w0 = plain[0].view(torch.float8_e4m3fn).float() if fp8 else plain[0].float()
+        want = x.float() @ w0.t()
+        best = None
+        for block in (256, 512, 1024):
+            for p1 in (1, 2, 4):
+                if (block // 64) % p1 or (n // 16) % p1:
+                    continue
+                for p2 in (2, 4, 6, 8):
+                    def call(a):
+                        return lambda: ops.gemv_layoutA_wapper(a, x, n, k, 1, 0, block, 1, p1, p2, scale, None)
+                    if not _gate(call(packed[0])(), want):
+                        continue
+                    us = _time_graph([call(a) for a in packed], iters)
+                    if best is None or us < best[0]:
+                        best = (us, block, 1, p1, p2)
+        print("%s %dx%d -> %s" % (table, n, k, best), file=sys.stderr)
+        rows.append("%d,%d,%d,%d,%d,%d" % (n, k, best[1], best[2], best[3], best[4]))
+        del plain, packed
+    return rows
+
+
+def scan_gemm(table, shapes, tokens, iters):
+    mode, dtype = GEMM_TABLES[table]
+    fp8 = mode == "fp8"
+    gen = torch.Generator(device="cuda").manual_seed(2025)
+    rows = []
+    for n, k in shapes:
+        plain = _weights(n, k, dtype, fp8, _copies(n * k * (1 if fp8 else 2)), gen)
+        packed = [ops.pack_layout_a(w) for w in plain]
+        w0 = plain[0].view(torch.float8_e4m3fn).float() if fp8 else plain[0].float()
+        scale = torch.ones((n // 128, k // 128), dtype=torch.float32, device="cuda") if fp8 else None
+        for m in tokens:
+            if mode in ("continuous", "native") and m % 16:
+                continue
+            b = torch.randn((m, k), generator=gen, device="cuda").to(dtype)
+            want = b.float() @ w0.t()
+            b_in = ops.layoutB(b) if mode in ("continuous", "native") else b
+            best = None
+            for p1 in (1, 2, 4):
+                if (n // 16) % p1:
+                    continue
+                for p2 in (1, 2, 4, 8, 16):
+                    def call(a):
+                        if mode == "rowmajor":
+                            return lambda: ops.gemm_layoutA_wapper(a, b_in, n, m, k, 1, 0, p1, p2, 1, 1, None)
+                        if mode == "fp8":
+                            return lambda: ops.gemm_layoutA_soft_fp8_wapper(a, scale, b_in, n, m, k, 1, 0, p1, p2, 1, 1,
+                                                                            None)
+                        if mode == "continuous":
+                            return lambda: ops.gemm_layoutAB_ContinuousC_wapper(a, b_in, n, m, k, 1, 0, p1, p2, 1, 1, None)
+                        return lambda: ops.gemm_layoutABC_wapper(a, b_in, n, m, k, 1, 0, p1, p2, 1, 1, None)
+                    got = call(packed[0])()
+                    if mode == "native":
+                        got = ops.reLayoutC(got)
+                    if not _gate(got, want):
+                        continue
+                    us = _time_graph([call(a) for a in packed], iters)
+                    if best is None or us < best[0]:
+                        best = (us, 1, p1, p2, 1)
+            print("%s %dx%d M=%d -> %s" % (table, n, k, m, best), file=sys.stderr)
+            rows.append("%d,%d,%d,%d,%d,%d,%d" % (n, m, k, best[1], best[2], best[3], best[4]))
+        del plain, packed
+    return rows
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("table", choices=list(GEMV_TABLES) + list(GEMM_TABLES) + ["all"])
+    ap.add_argument("--shapes", default=None, help="comma separated MxK weight shapes, e.g. 4096x4096,11008x4096")
+    ap.add_argument("--tokens", default=None, help="comma separated token counts for the GEMM tables")
+    ap.add_argument("--iters", type=int, default=40)
+    ap.add_argument("--update", action="store_true", help="append the rows to the packaged csv")
+    args = ap.parse_args()
+    tables = (list(GEMV_TABLES) + list(GEMM_TABLES)) if args.table == "all" else [args.table]
+    for table in tables:
+        shapes = DEFAULT_SHAPES[table] if args.shapes is None else \
+            [tuple(int(v) for v in s.split("x")) for s in args.shapes.split(",")]
+        if table in GEMV_TABLES:
+            rows = scan_gemv(table, shapes, args.iters)
+            header = "m,k,BLOCK_DIM_X,KernelId,KernelParam1,KernelParam2"
+        else:
+            tokens = DEFAULT_TOKENS[table] if args.tokens is None else [int(v) for v in args.tokens.split(",")]
+            rows = scan_gemm(table, shapes, tokens, args.iters)
+            header = "m,n,k,kernelId,kernelParam1,kernelParam2,kernelParam3"
+        if args.update:
+            path = arg_selector.selector(table).path()
+            with open(path, "a") as f:
+                f.write("\n".join(rows) + "\n")
+        else:
+            path = "%s_scan_best_args.csv" % table
+            with open(path, "w") as f:
+                f.write(header + "\n" + "\n".join(rows) + "\n")
+        print("wrote %d rows to %s" % (len(rows), path), file=sys.stderr)
+
+
+if __name__ == "__main__":
+    main()
