@@ -164,8 +164,8 @@ def main():
                 w1 = w1.to(torch.float8_e4m3fn).view(torch.uint8)
                 w2 = (torch.randn((E, H, I), generator=gen, device=dev) * 16).clamp_(-448, 448)
                 w2 = w2.to(torch.float8_e4m3fn).view(torch.uint8)
-                s1 = torch.full((E, 2 * I // 128, H // 128), 0.02 / 16, dtype=torch.float32, device=dev)
-                s2 = torch.full((E, H // 128, I // 128), 0.02 / 16, dtype=torch.float32, device=dev)
+                s1 = torch.ones((E, 2 * I // 128, H // 128), dtype=torch.float32, device=dev)
+                s2 = torch.ones((E, H // 128, I // 128), dtype=torch.float32, device=dev)
                 moe_w[key] = (w1, w2, s1, s2)
             else:
                 w1 = (torch.randn((E, 2 * I, H), generator=gen, device=dev) * 0.02).to(torch.bfloat16)

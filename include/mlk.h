@@ -46,6 +46,10 @@ extern "C" {
 
 int mlk_version(void);
 const char *mlk_last_error(void);
+/* Experiment switches for the tuning scripts (process-wide, not thread-safe):
+ * id 0 = rotate the k-tile visiting order of the narrow GeMM per row tile (default 1).
+ * No counterpart in the reference. */
+void mlk_set_tunable(int id, int value);
 
 /* ------------------------------------------------------------------ relayout
  * Pure permutations of 16-byte (16-bit elements) or 8-byte (fp8) granules;

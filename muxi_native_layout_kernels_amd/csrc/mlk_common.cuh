@@ -98,10 +98,68 @@ __device__ __forceinline__ void fp8x4_to_bf16x4(uint32_t w, float scale, uint32_
     hi = __builtin_amdgcn_perm(__float_as_uint(b1), __float_as_uint(b0), 0x07060302u);
 }
 
+// Power-of-two scales (sign 0, mantissa 0, normal exponent) take a shorter road: the scaled
+// converter v_cvt_scalef32_pk_bf16_fp8 multiplies by 2^(exponent of the scale) while widening
+// two bytes to packed bf16, which is exact - the same bits as the general path - at a fifth of
+// the VALU work.  The test is on a wave-uniform value, so the branch is scalar.
+__device__ __forceinline__ bool scale_is_pow2(float scale) {
+    const uint32_t b = __float_as_uint(scale);
+    return (b & 0x807fffffu) == 0u && b != 0u && b != 0x7f800000u;
+}
+__device__ __forceinline__ void fp8x4_to_bf16x4_pow2(uint32_t w, float scale, uint32_t &lo, uint32_t &hi) {
+    lo = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)w, scale, false));
+    hi = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8((int)w, scale, true));
+}
+
+// One row of block scales (one fp32 per 128 k) kept in registers: lane l of register i holds
+// the scale of k block 64 i + l.  scale_at() fetches a wave-uniform entry with v_readlane, so
+// the streaming loops never wait on memory for a scale.  Covers K <= 32768.
+constexpr int kMaxScaleK = 32768;
+struct ScaleRow {
+    float v[4];
+};
+__device__ __forceinline__ ScaleRow load_scale_row(const float *row, int cols, int lane) {
+    ScaleRow s;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        int idx = lane + 64 * i;
+        s.v[i] = (row != nullptr && idx < cols) ? row[idx] : 1.f;
+    }
+    return s;
+}
+__device__ __forceinline__ float scale_at(const ScaleRow &s, int kblock /* wave-uniform */) {
+    const int hi = kblock >> 6;
+    float x = hi == 0 ? s.v[0] : (hi == 1 ? s.v[1] : (hi == 2 ? s.v[2] : s.v[3]));
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), kblock & 63));
+}
+
 // 64-lane xor shuffle of an fp32 through the LDS crossbar (no LDS memory used).
 __device__ __forceinline__ float lane_xor(float v, int mask) {
     int lane = __lane_id();
     return __int_as_float(__builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, __float_as_int(v)));
+}
+
+// Partial sums exchanged between workgroups of one kernel.  The L2 caches of the eight XCDs are
+// not coherent with each other for ordinary accesses; agent-scope atomic accesses are (they are
+// issued write-through / always-miss), and unlike an agent-scope fence they do not write back or
+// invalidate a whole L2.  64-bit relaxed atomics carry two floats each.
+__device__ __forceinline__ void st_agent_f32x4(f32x4 *p, f32x4 v) {
+    uint64_t *q = reinterpret_cast<uint64_t *>(p);
+    uint64_t lo = (uint64_t)__float_as_uint(v[0]) | ((uint64_t)__float_as_uint(v[1]) << 32);
+    uint64_t hi = (uint64_t)__float_as_uint(v[2]) | ((uint64_t)__float_as_uint(v[3]) << 32);
+    __hip_atomic_store(q, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(q + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ f32x4 ld_agent_f32x4(const f32x4 *p) {
+    const uint64_t *q = reinterpret_cast<const uint64_t *>(p);
+    uint64_t lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint64_t hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    f32x4 v;
+    v[0] = __uint_as_float((uint32_t)lo);
+    v[1] = __uint_as_float((uint32_t)(lo >> 32));
+    v[2] = __uint_as_float((uint32_t)hi);
+    v[3] = __uint_as_float((uint32_t)(hi >> 32));
+    return v;
 }
 
 __device__ __forceinline__ u32x4 ld_global_u32x4(const void *p) { return *reinterpret_cast<const u32x4 *>(p); }

@@ -25,6 +25,10 @@ namespace mlk {
 
 constexpr size_t kCounterBytes = 64 * 1024;
 
+// Experiment switches (mlk_set_tunable): [0] rotate the k-tile order per row tile,
+// [1] stage row-major activations through LDS.
+static int g_tunable[8] = {1, 1, 0, 0, 0, 0, 0, 0};
+
 struct GemmArgs {
     const uint8_t *A;
     const uint16_t *B;
@@ -38,12 +42,13 @@ struct GemmArgs {
     int cb0;             // first 16-token block of this launch
     int N, K;
     int WK, SK;
+    int rotate;
     float alpha;
 };
 
-template <class T, bool FP8, int CB, int R, int BMODE, int CMODE, int U>
+template <class T, bool FP8, int CB, int R, int BMODE, int CMODE, int U, bool STAGE>
 __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel(GemmArgs p) {
-    extern __shared__ f32x4 red[];  // [WK][R*CB][64]
+    extern __shared__ f32x4 red[];  // [WK][R*CB][64]; the staged variant first uses it for two activation windows
     __shared__ int s_last;
 
     const int lane = threadIdx.x & 63;
@@ -65,20 +70,23 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel
     for (int r = 0; r < R; ++r) abase[r] = p.A + (size_t)(rg0 + r) * p.K * 16 * WBYTES;
 
     // activation fragment source for this lane
+    // Lanes whose token does not exist read the last real token instead: column c of the
+    // product depends only on column c of the activations, and those columns are never stored.
     const uint16_t *bptr[CB];
-    bool bok[CB];
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
         if (BMODE == MLK_B_NATIVE) {
             bptr[cb] = p.B + ((size_t)(p.cb0 + cb) * 64 + lane) * 8;
-            bok[cb] = true;
         } else {
-            int tok = (p.cb0 + cb) * 16 + r16;
-            bok[cb] = tok < p.M_total;
-            bptr[cb] = p.B + (size_t)(bok[cb] ? tok : 0) * p.K + q * 8;
+            int tok = min((p.cb0 + cb) * 16 + r16, p.M_total - 1);
+            bptr[cb] = p.B + (size_t)tok * p.K + q * 8;
         }
     }
     const size_t bstep = (BMODE == MLK_B_NATIVE) ? (size_t)mb_total * 512 : 32;  // elements per k tile
+
+    // the R row groups of a wave (R divides 8, rg0 is a multiple of R) share one row of block scales
+    ScaleRow srow;
+    if (FP8) srow = load_scale_row(p.scale ? p.scale + (size_t)(rg0 >> 3) * scale_cols : nullptr, scale_cols, lane);
 
     f32x4 acc[R][CB];
 #pragma unroll
@@ -95,13 +103,10 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
-            if (FP8) sc[slot][r] = p.scale ? p.scale[((rg0 + r) >> 3) * scale_cols + (kt >> 2)] : 1.f;
+            if (FP8) sc[slot][r] = scale_at(srow, kt >> 2);
         }
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-            if (bok[cb]) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * bstep);
-            else bf[slot][cb] = u32x4{0u, 0u, 0u, 0u};
-        }
+        for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * bstep);
     };
     auto consume = [&](int slot) {
         u32x4 a[R], b[CB];
@@ -114,46 +119,127 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) acc[r][cb] = T::mfma(a[r], b[cb], acc[r][cb]);
     };
-    // The wave visits its k tiles in a rotated order that differs from row tile to row tile:
-    // workgroups that run side by side then read different parts of the (small, shared)
-    // activation matrix at any moment instead of all hitting the same cache lines.
-    int jcur = nt > 0 ? (int)(((unsigned)rt * 2654435761u >> 7) % (unsigned)nt) : 0;
-    auto next_tile = [&]() {
-        int t = tbeg + wave + jcur * p.WK;
-        jcur = (jcur + 1 == nt) ? 0 : jcur + 1;
-        return t;
-    };
+    if constexpr (STAGE) {
+        // Row-major activations, staged: in step j the WK waves work on the window of WK
+        // consecutive k tiles [tbeg + w*WK, +WK).  The workgroup fetches the window's
+        // activations with row-contiguous 16-byte loads (WK*64 bytes per token), one step
+        // ahead, and leaves them in LDS in MFMA fragment order (two buffers, one barrier per
+        // step); each wave then reads its own tile's fragments with ds_read_b128.  Fragment
+        // rows are padded (68 granules per tile, 17 per k-octet) against bank conflicts.
+        u32x4 *win = reinterpret_cast<u32x4 *>(red);
+        const int win_granules = p.WK * CB * 68;
+        const int nwin = (tend - tbeg) / p.WK;            // exact: the host only stages when WK divides the slice
+        const int cols = p.WK * 4;                        // 16-byte granules per token in a window
+        const int sh = __builtin_ctz(cols);
+        int rot = (nwin > 0 && p.rotate) ? (int)(((unsigned)rt * 2654435761u >> 7) % (unsigned)nwin) : 0;
+        int w_stage = rot, w_issue = rot;
+        auto advance = [&](int &w) {
+            int cur = w;
+            w = (w + 1 == nwin) ? 0 : w + 1;
+            return cur;
+        };
+        u32x4 breg[CB];
+        auto stage_load = [&]() {
+            const int tile0 = tbeg + advance(w_stage) * p.WK;
+#pragma unroll
+            for (int i = 0; i < CB; ++i) {
+                const int g = threadIdx.x + i * blockDim.x;
+                const int row = g >> sh, colg = g & (cols - 1);
+                const int tok = min(p.cb0 * 16 + row, p.M_total - 1);
+                breg[i] = ld_global_u32x4(p.B + (size_t)tok * p.K + (size_t)tile0 * 32 + colg * 8);
+            }
+        };
+        auto stage_store = [&](int buf) {
+#pragma unroll
+            for (int i = 0; i < CB; ++i) {
+                const int g = threadIdx.x + i * blockDim.x;
+                const int row = g >> sh, colg = g & (cols - 1);
+                win[buf * win_granules + ((colg >> 2) * CB + (row >> 4)) * 68 + (colg & 3) * 17 + (row & 15)] = breg[i];
+            }
+        };
+        auto issue_a = [&](int slot) {
+            const int kt = tbeg + advance(w_issue) * p.WK + wave;
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
+                if (FP8) sc[slot][r] = scale_at(srow, kt >> 2);
+            }
+        };
+        auto step = [&](int slot, int buf, bool do_stage, bool do_issue) {
+            if (do_stage) stage_load();
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = win[buf * win_granules + (wave * CB + cb) * 68 + q * 17 + r16];
+            consume(slot);
+            if (do_issue) issue_a(slot);
+            __builtin_amdgcn_sched_barrier(0);
+            if (do_stage) stage_store(buf ^ 1);
+            __syncthreads();
+        };
+        static_assert(U % 2 == 0, "the staged loop alternates two LDS buffers inside a U-step unroll");
+        if (nwin > 0) {
+            stage_load();
+            stage_store(0);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < nwin) issue_a(u);
+            __syncthreads();
+            int j = 0;
+            for (; j + 2 * U <= nwin; j += U) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) step(u, u & 1, true, true);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (j + u < nwin) step(u, u & 1, j + u + 1 < nwin, j + u + U < nwin);
+            j += U;
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (j + u < nwin) step(u, u & 1, j + u + 1 < nwin, false);
+        }
+        __syncthreads();   // the windows are dead; the same LDS now serves the wave fold
+    } else {
+        // The wave visits its k tiles in a rotated order that differs from row tile to row tile:
+        // workgroups that run side by side then read different parts of the (small, shared)
+        // activation matrix at any moment instead of all hitting the same cache lines.
+        int jcur = (nt > 0 && p.rotate) ? (int)(((unsigned)rt * 2654435761u >> 7) % (unsigned)nt) : 0;
+        auto next_tile = [&]() {
+            int t = tbeg + wave + jcur * p.WK;
+            jcur = (jcur + 1 == nt) ? 0 : jcur + 1;
+            return t;
+        };
 
-    // Register ring of U k-tiles; the steady-state loop is branch-free so the loads stay
-    // U tiles deep in flight.
-    if (nt >= U) {
-#pragma unroll
-        for (int u = 0; u < U; ++u) issue(u, next_tile());
-        int i = 0;
-        for (; i + 2 * U <= nt; i += U) {
-#pragma unroll
+        // Register ring of U k-tiles; the steady-state loop is branch-free so the loads stay
+        // U tiles deep in flight.
+        if (nt >= U) {
+    #pragma unroll
+            for (int u = 0; u < U; ++u) issue(u, next_tile());
+            int i = 0;
+            for (; i + 2 * U <= nt; i += U) {
+    #pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    consume(u);
+                    issue(u, next_tile());
+                    __builtin_amdgcn_sched_barrier(0);  // keep each refill right behind its consume
+                }
+            }
+            const int rem = nt - i - U;
+    #pragma unroll
             for (int u = 0; u < U; ++u) {
                 consume(u);
-                issue(u, next_tile());
-                __builtin_amdgcn_sched_barrier(0);  // keep each refill right behind its consume
+                if (u < rem) issue(u, next_tile());
             }
+    #pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < rem) consume(u);
+        } else {
+    #pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < nt) issue(u, next_tile());
+    #pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < nt) consume(u);
         }
-        const int rem = nt - i - U;
-#pragma unroll
-        for (int u = 0; u < U; ++u) {
-            consume(u);
-            if (u < rem) issue(u, next_tile());
-        }
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-            if (u < rem) consume(u);
-    } else {
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-            if (u < nt) issue(u, next_tile());
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-            if (u < nt) consume(u);
+
     }
 
     constexpr int NTILE = R * CB;
@@ -192,7 +278,7 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) part[part_at(sk, r * CB + cb)] = acc[r][cb];
+            for (int cb = 0; cb < CB; ++cb) st_agent_f32x4(&part[part_at(sk, r * CB + cb)], acc[r][cb]);
     } else {
         // fold the WK waves through LDS in wave order; wave w then owns tiles j = w, w + WK, ...
 #pragma unroll
@@ -204,26 +290,28 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel
             f32x4 v = red[j * 64 + lane];
             for (int w = 1; w < p.WK; ++w) v += red[(w * NTILE + j) * 64 + lane];
             if (p.SK == 1) epilogue(j, v);
-            else part[part_at(sk, j)] = v;
+            else st_agent_f32x4(&part[part_at(sk, j)], v);
         }
         if (p.SK == 1) return;
     }
 
-    // ---- K split across workgroups: the partial is published, the last workgroup to arrive
-    // for this row tile folds all slices in slice order
-    __threadfence();
+    // ---- K split across workgroups: the partial is published with agent-coherent stores, the
+    // last workgroup to arrive for this row tile folds all slices in slice order.  Every wave
+    // waits for its own stores to be acknowledged before the barrier; the arrival counter is
+    // bumped after the barrier, so a workgroup that sees SK-1 earlier arrivals can read all
+    // partials.
+    __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (threadIdx.x == 0) {
-        int prev = atomicAdd(&p.counters[rt], 1);
+        int prev = __hip_atomic_fetch_add(&p.counters[rt], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         s_last = (prev == p.SK - 1);
-        if (s_last) p.counters[rt] = 0;
+        if (s_last) __hip_atomic_store(&p.counters[rt], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
     if (!s_last) return;
-    __threadfence();
     for (int j = wave; j < NTILE; j += p.WK) {
         f32x4 v = {0.f, 0.f, 0.f, 0.f};
-        for (int s = 0; s < p.SK; ++s) v += part[part_at(s, j)];
+        for (int s = 0; s < p.SK; ++s) v += ld_agent_f32x4(&part[part_at(s, j)]);
         epilogue(j, v);
     }
 }
@@ -236,7 +324,20 @@ static int launch(const GemmArgs &p, hipStream_t s) {
     int row_tiles = (q.N / 16) / R;
     int grid = row_tiles * q.SK;
     size_t lds = q.WK > 1 ? (size_t)q.WK * R * CB * 1024 : 0;
-    gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, U><<<grid, q.WK * 64, lds, s>>>(q);
+    if constexpr (BMODE == MLK_B_ROWMAJOR) {
+        // stage row-major activations through LDS when every K slice is a whole number of WK-tile windows
+        const int tiles_total = q.K / 32;
+        const int tiles_per = (tiles_total + q.SK - 1) / q.SK;
+        const size_t win_bytes = (size_t)2 * q.WK * CB * 68 * 16;
+        if (g_tunable[1] && q.WK >= 2 && tiles_total % q.SK == 0 && tiles_per % q.WK == 0 && win_bytes <= 48 * 1024) {
+            constexpr int US = (R * CB >= 8) ? 2 : 4;
+            if (win_bytes > lds) lds = win_bytes;
+            gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, US, true><<<grid, q.WK * 64, lds, s>>>(q);
+            MLK_LAUNCH_CHECK();
+            return MLK_OK;
+        }
+    }
+    gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, U, false><<<grid, q.WK * 64, lds, s>>>(q);
     MLK_LAUNCH_CHECK();
     return MLK_OK;
 }
@@ -269,6 +370,10 @@ static int launch_modes(const GemmArgs &p, int b_mode, int c_mode, int R, int CB
 
 using namespace mlk;
 
+extern "C" void mlk_set_tunable(int id, int value) {
+    if (id >= 0 && id < 8) g_tunable[id] = value;
+}
+
 extern "C" size_t mlk_gemm_counter_bytes(void) { return kCounterBytes; }
 
 extern "C" size_t mlk_gemm_workspace_bytes(int m, int n, int p1, int p3) {
@@ -299,6 +404,7 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
     const bool fp8 = a_kind == MLK_FP8_E4M3;
     if (fp8) {
         MLK_REQUIRE(x_kind == MLK_BF16, "gemm: soft-FP8 weights need bf16 activations");
+        MLK_REQUIRE(k <= kMaxScaleK, "gemm: soft-FP8 supports K <= 32768");
     } else {
         MLK_REQUIRE(a_kind == x_kind, "gemm: weights and activations must have the same 16-bit type");
         MLK_REQUIRE(scale == nullptr, "gemm: a scale matrix is only meaningful for soft-FP8 weights");
@@ -330,6 +436,7 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
     g.WK = wk;
     g.SK = sk;
     g.alpha = alpha;
+    g.rotate = g_tunable[0];
     hipStream_t s = (hipStream_t)stream;
     // weight passes of at most 64 tokens
     for (int c0 = 0; c0 < m; c0 += 64) {

@@ -42,8 +42,13 @@ __device__ __forceinline__ u32x4 weight_operand(const WeightFrag<FP8> &f, float 
     if constexpr (FP8) {
         u32x4 o;
         uint32_t a, b, c, d;
-        fp8x4_to_bf16x4(f.v[0], scale, a, b);
-        fp8x4_to_bf16x4(f.v[1], scale, c, d);
+        if (scale_is_pow2(scale)) {
+            fp8x4_to_bf16x4_pow2(f.v[0], scale, a, b);
+            fp8x4_to_bf16x4_pow2(f.v[1], scale, c, d);
+        } else {
+            fp8x4_to_bf16x4(f.v[0], scale, a, b);
+            fp8x4_to_bf16x4(f.v[1], scale, c, d);
+        }
         o[0] = a; o[1] = b; o[2] = c; o[3] = d;
         return o;
     } else {

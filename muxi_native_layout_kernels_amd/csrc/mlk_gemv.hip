@@ -49,6 +49,9 @@ __global__ void __launch_bounds__(1024)
 #pragma unroll
         for (int m = 0; m < M; ++m) acc[a][m] = 0.f;
 
+    ScaleRow srow;
+    if (FP8) srow = load_scale_row(scale ? scale + (size_t)((active ? rg : 0) >> 3) * scale_cols : nullptr, scale_cols, lane);
+
     const u32x4 *arow = reinterpret_cast<const u32x4 *>(A) + (size_t)(active ? rg : 0) * tiles_total * 64 + lane;
     const int stride = WK * 64;                   // u32x4 units between this wave's tiles
 
@@ -65,7 +68,7 @@ __global__ void __launch_bounds__(1024)
         float sc[U];
         auto issue = [&](int u, int j) {          // j = index among this wave's tiles in the window
             buf[u] = ld_stream_u32x4(ap + (size_t)j * stride);
-            if (FP8) sc[u] = scale ? scale[(rg >> 3) * scale_cols + ((t0 + ks + j * WK) >> 1)] : 1.f;
+            if (FP8) sc[u] = scale_at(srow, (t0 + ks + j * WK) >> 1);
         };
         auto consume = [&](int u, int j) {
             u32x4 cur = buf[u];
@@ -73,10 +76,17 @@ __global__ void __launch_bounds__(1024)
             if (FP8) {
                 float s = sc[u];
                 uint32_t w0[4], w1[4];
-                fp8x4_to_bf16x4(cur[0], s, w0[0], w0[1]);
-                fp8x4_to_bf16x4(cur[1], s, w0[2], w0[3]);
-                fp8x4_to_bf16x4(cur[2], s, w1[0], w1[1]);
-                fp8x4_to_bf16x4(cur[3], s, w1[2], w1[3]);
+                if (scale_is_pow2(s)) {
+                    fp8x4_to_bf16x4_pow2(cur[0], s, w0[0], w0[1]);
+                    fp8x4_to_bf16x4_pow2(cur[1], s, w0[2], w0[3]);
+                    fp8x4_to_bf16x4_pow2(cur[2], s, w1[0], w1[1]);
+                    fp8x4_to_bf16x4_pow2(cur[3], s, w1[2], w1[3]);
+                } else {
+                    fp8x4_to_bf16x4(cur[0], s, w0[0], w0[1]);
+                    fp8x4_to_bf16x4(cur[1], s, w0[2], w0[3]);
+                    fp8x4_to_bf16x4(cur[2], s, w1[0], w1[1]);
+                    fp8x4_to_bf16x4(cur[3], s, w1[2], w1[3]);
+                }
 #pragma unroll
                 for (int m = 0; m < M; ++m) {
                     u32x4 xv = xs[m * (KC >> 3) + xg];
@@ -247,6 +257,7 @@ extern "C" int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, i
     if (a_kind == MLK_FP8_E4M3) {
         MLK_REQUIRE(x_kind == MLK_BF16, "gemv: soft-FP8 weights need bf16 activations");
         MLK_REQUIRE(k % 64 == 0, "gemv: soft-FP8 needs K % 64 == 0");
+        MLK_REQUIRE(k <= kMaxScaleK, "gemv: soft-FP8 supports K <= 32768");
         return launch_m<BF16, true>(m, a, x, y, n, k, alpha, bias, scale, block_dim_x, p1, p2, s);
     }
     MLK_REQUIRE(a_kind == x_kind, "gemv: weights and activations must have the same 16-bit type");

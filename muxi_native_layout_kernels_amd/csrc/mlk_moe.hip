@@ -282,18 +282,78 @@ struct MoeArgs {
     const int32_t *sorted;    // [T*K + E*15]
     const MoeTask *tasks;
     const int32_t *n_tasks;
-    int T, K, H, I, SB, n_pairs, WK;
+    const int32_t *topk_ids;  // [T*K], read by the decode variants that align in-kernel
+    const int32_t *experts_map;
+    int T, K, H, I, SB, n_pairs, WK, E;
 };
 
+// Decode-sized batches (T*K <= 64 pairs): every workgroup rebuilds the tiny alignment itself
+// from the routing table instead of waiting for a separate alignment launch.  One wave walks
+// the distinct experts in order of first appearance; an expert's pairs keep ascending order and
+// fill 16-slot blocks (block id = task id), padded with the sentinel n_pairs.
+constexpr int kDecodePairs = 64;
+struct DecodeTables {
+    MoeTask tasks[kDecodePairs];
+    int sorted[kDecodePairs * 16];
+    int n_tasks;
+};
+__device__ __forceinline__ void build_decode_tables(DecodeTables &t, const int32_t *topk_ids,
+                                                    const int32_t *experts_map, int n_pairs, int E, int lane) {
+    int e = -1;
+    if (lane < n_pairs) {
+        e = topk_ids[lane];
+        if (experts_map) e = experts_map[e];
+        if (e < 0 || e >= E) e = -1;
+    }
+    unsigned long long todo = __ballot(e >= 0);
+    int nt = 0;
+    while (todo) {
+        const int leader = __ffsll((long long)todo) - 1;
+        const int le = __shfl(e, leader);
+        const unsigned long long same = __ballot(e == le);
+        const int cnt = __popcll(same);
+        const int nb = (cnt + 15) >> 4;
+        if (e == le) {
+            const int rank = __popcll(same & ((1ull << lane) - 1ull));
+            t.sorted[nt * 16 + rank] = lane;
+        }
+        if (lane < nb * 16 - cnt) t.sorted[nt * 16 + cnt + lane] = n_pairs;
+        if (lane < nb) {
+            MoeTask tk;
+            tk.expert = le;
+            tk.block0 = nt + lane;
+            tk.nblocks = 1;
+            tk.pad = 0;
+            t.tasks[nt + lane] = tk;
+        }
+        nt += nb;
+        todo &= ~same;
+    }
+    if (lane == 0) t.n_tasks = nt;
+}
+
 // gate/up projection with SiLU(gate) * up, one task per blockIdx.y
-template <class T, bool FP8, int CB, int P, int U>
+template <class T, bool FP8, int CB, int P, int U, bool INLINE>
 __global__ void __launch_bounds__(max_threads_for_tiles(2 * P * CB)) moe_gate_up_kernel(MoeArgs p) {
     extern __shared__ f32x4 red[];  // [WK][2P*CB][64]
-    const int task = blockIdx.y;
-    if (task >= p.n_tasks[0]) return;
-    const MoeTask tk = p.tasks[task];
+    __shared__ DecodeTables dec;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int task = blockIdx.y;
+    const MoeTask *tasks = p.tasks;
+    const int32_t *sorted = p.sorted;
+    int n_tasks;
+    if (INLINE) {
+        if (wave == 0) build_decode_tables(dec, p.topk_ids, p.experts_map, p.n_pairs, p.E, lane);
+        __syncthreads();
+        tasks = dec.tasks;
+        sorted = dec.sorted;
+        n_tasks = dec.n_tasks;
+    } else {
+        n_tasks = p.n_tasks[0];
+    }
+    if (task >= n_tasks) return;
+    const MoeTask tk = tasks[task];
     const int q = lane >> 4, r16 = lane & 15;
     const int g0 = blockIdx.x * P;
     constexpr int WB = FP8 ? 1 : 2;
@@ -304,21 +364,29 @@ __global__ void __launch_bounds__(max_threads_for_tiles(2 * P * CB)) moe_gate_up
     const int scale_cols = p.H >> 7;
 
     const uint8_t *abase[R];
-    int srow[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         int rg = (r & 1) * groups_i + g0 + (r >> 1);
         abase[r] = p.W1 + (size_t)tk.expert * slab + (size_t)rg * p.H * 16 * WB;
-        srow[r] = (tk.expert * (2 * p.I >> 7) + (rg >> 3)) * scale_cols;
     }
+    // block scales of the gate rows and of the up rows (the P pairs of a wave share a 128-row block)
+    ScaleRow srows[2];
+    if (FP8) {
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            int rg = h * groups_i + g0;
+            srows[h] = load_scale_row(
+                p.S1 ? p.S1 + ((size_t)tk.expert * (2 * p.I >> 7) + (rg >> 3)) * scale_cols : nullptr, scale_cols, lane);
+        }
+    }
+    // Padding slots and blocks beyond the task read token 0: their columns of the product are
+    // written to padding rows of the intermediate (or not at all) and never reach the output.
     const uint16_t *bptr[CB];
-    bool bok[CB];
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
         int id = p.n_pairs;
-        if (cb < tk.nblocks) id = p.sorted[(tk.block0 + cb) * 16 + r16];
-        bok[cb] = id < p.n_pairs;
-        bptr[cb] = p.X + (size_t)(bok[cb] ? id / p.K : 0) * p.H + q * 8;
+        if (cb < tk.nblocks) id = sorted[(tk.block0 + cb) * 16 + r16];
+        bptr[cb] = p.X + (size_t)(id < p.n_pairs ? id / p.K : 0) * p.H + q * 8;
     }
 
     f32x4 acc[R][CB];
@@ -335,13 +403,10 @@ __global__ void __launch_bounds__(max_threads_for_tiles(2 * P * CB)) moe_gate_up
 #pragma unroll
         for (int r = 0; r < R; ++r) {
             wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
-            if (FP8) sc[slot][r] = p.S1 ? p.S1[srow[r] + (kt >> 2)] : 1.f;
+            if (FP8) sc[slot][r] = scale_at(srows[r & 1], kt >> 2);
         }
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb) {
-            if (bok[cb]) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * 32);
-            else bf[slot][cb] = u32x4{0u, 0u, 0u, 0u};
-        }
+        for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * 32);
     };
     auto consume = [&](int slot) {
         u32x4 a[R], b[CB];
@@ -412,12 +477,23 @@ __global__ void __launch_bounds__(max_threads_for_tiles(2 * P * CB)) moe_gate_up
     }
 }
 
-// down projection over all tasks, routing weights and the sum over a token's experts in LDS
-template <class T, bool FP8, int CB, int R, int U>
+// Down projection over all tasks, routing weights and the sum over a token's experts in LDS.
+//
+// The workgroup owns R row groups of the output and walks the task list in rounds.  In a round
+// the WK waves are dealt out to up to WK tasks (WK / g waves per task, each taking every
+// (WK/g)-th k tile of that task's expert), so the weight streams of all the round's experts are
+// in flight together and the pipeline drains once per round, not once per expert.  The fold and
+// the routing-weighted scatter into the fp32 output tile then run task by task in list order, so
+// the summation order of a token's experts is fixed.
+template <class T, bool FP8, int CB, int R, int U, bool INLINE>
 __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(MoeArgs p) {
     extern __shared__ f32x4 red[];  // [WK][R*CB][64] then the fp32 output tile [T][16R]
+    __shared__ DecodeTables dec;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const MoeTask *tasks = p.tasks;
+    const int32_t *sorted = p.sorted;
+    if (INLINE && wave == 0) build_decode_tables(dec, p.topk_ids, p.experts_map, p.n_pairs, p.E, lane);
     const int q = lane >> 4, r16 = lane & 15;
     const int rg0 = blockIdx.x * R;
     constexpr int WB = FP8 ? 1 : 2;
@@ -431,20 +507,34 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
     for (int i = threadIdx.x; i < p.T * yrows; i += blockDim.x) ytile[i] = 0.f;
     __syncthreads();
 
-    const int n_tasks = p.n_tasks[0];
-    const int nt = (wave < tiles_total) ? (tiles_total - wave + p.WK - 1) / p.WK : 0;
-    for (int task = 0; task < n_tasks; ++task) {
-        const MoeTask tk = p.tasks[task];
+    int n_tasks;
+    if (INLINE) {
+        tasks = dec.tasks;
+        sorted = dec.sorted;
+        n_tasks = dec.n_tasks;
+    } else {
+        n_tasks = p.n_tasks[0];
+    }
+    for (int base = 0; base < n_tasks;) {
+        const int g = min(p.WK, n_tasks - base);      // tasks of this round
+        const int wpt = p.WK / g;                     // waves per task
+        const int tl = wave / wpt;                    // this wave's task inside the round
+        const int ks = wave - tl * wpt;               // and its k slice
+        const bool busy = tl < g;
+        const MoeTask tk = tasks[base + (busy ? tl : 0)];
+        const int nt = (busy && ks < tiles_total) ? (tiles_total - ks + wpt - 1) / wpt : 0;
+
         const uint8_t *abase[R];
-        int srow[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            abase[r] = p.W2 + (size_t)tk.expert * slab + (size_t)(rg0 + r) * p.I * 16 * WB;
-            srow[r] = (tk.expert * (p.H >> 7) + ((rg0 + r) >> 3)) * scale_cols;
-        }
+        for (int r = 0; r < R; ++r) abase[r] = p.W2 + (size_t)tk.expert * slab + (size_t)(rg0 + r) * p.I * 16 * WB;
+        ScaleRow srow;
+        if (FP8)
+            srow = load_scale_row(
+                p.S2 ? p.S2 + ((size_t)tk.expert * (p.H >> 7) + (rg0 >> 3)) * scale_cols : nullptr, scale_cols, lane);
         const uint16_t *bptr[CB];
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb) bptr[cb] = p.Hbuf + ((size_t)(tk.block0 + cb) * 64 + lane) * 8;
+        for (int cb = 0; cb < CB; ++cb)
+            bptr[cb] = p.Hbuf + ((size_t)(tk.block0 + (cb < tk.nblocks ? cb : 0)) * 64 + lane) * 8;
         const size_t bstep = (size_t)p.SB * 512;
 
         f32x4 acc[R][CB];
@@ -459,13 +549,10 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
 #pragma unroll
             for (int r = 0; r < R; ++r) {
                 wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
-                if (FP8) sc[slot][r] = p.S2 ? p.S2[srow[r] + (kt >> 2)] : 1.f;
+                if (FP8) sc[slot][r] = scale_at(srow, kt >> 2);
             }
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) {
-                if (cb < tk.nblocks) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * bstep);
-                else bf[slot][cb] = u32x4{0u, 0u, 0u, 0u};
-            }
+            for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * bstep);
         };
         auto consume = [&](int slot) {
             u32x4 a[R], b[CB];
@@ -479,7 +566,7 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
                 for (int cb = 0; cb < CB; ++cb) acc[r][cb] = T::mfma(a[r], b[cb], acc[r][cb]);
         };
         int jcur = 0;
-        auto next_tile = [&]() { return wave + (jcur++) * p.WK; };
+        auto next_tile = [&]() { return ks + (jcur++) * wpt; };
         if (nt >= U) {
 #pragma unroll
             for (int u = 0; u < U; ++u) issue(u, next_tile());
@@ -515,19 +602,24 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) red[(wave * NT + r * CB + cb) * 64 + lane] = acc[r][cb];
         __syncthreads();
-        for (int j = wave; j < NT; j += p.WK) {
-            const int r = j / CB, cb = j - r * CB;
-            if (cb >= tk.nblocks) continue;
-            const int id = p.sorted[(tk.block0 + cb) * 16 + r16];
-            if (id >= p.n_pairs) continue;
-            f32x4 v = red[j * 64 + lane];
-            for (int w = 1; w < p.WK; ++w) v += red[(w * NT + j) * 64 + lane];
-            const float wt = T::to_f32(p.wts[id]);
-            float *dst = ytile + (size_t)(id / p.K) * yrows + r * 16 + 4 * q;
+        // fold and scatter task by task (list order), tiles of one task spread over the waves
+        for (int t = 0; t < g; ++t) {
+            const MoeTask ft = tasks[base + t];
+            for (int j = wave; j < NT; j += p.WK) {
+                const int r = j / CB, cb = j - r * CB;
+                if (cb >= ft.nblocks) continue;
+                const int id = sorted[(ft.block0 + cb) * 16 + r16];
+                if (id >= p.n_pairs) continue;
+                f32x4 v = red[((t * wpt) * NT + j) * 64 + lane];
+                for (int w = 1; w < wpt; ++w) v += red[((t * wpt + w) * NT + j) * 64 + lane];
+                const float wt = T::to_f32(p.wts[id]);
+                float *dst = ytile + (size_t)(id / p.K) * yrows + r * 16 + 4 * q;
 #pragma unroll
-            for (int i = 0; i < 4; ++i) dst[i] += wt * v[i];
+                for (int i = 0; i < 4; ++i) dst[i] += wt * v[i];
+            }
+            __syncthreads();
         }
-        __syncthreads();
+        base += g;
     }
 
     for (int i = threadIdx.x; i < p.T * yrows; i += blockDim.x) {
@@ -549,7 +641,8 @@ static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; 
 static size_t carve(uint8_t *base, int tc, int E, int K, int inter, MoeWorkspace *ws) {
     const int n_pairs = tc * K;
     const int max_padded = n_pairs + E * 15;
-    const int max_blocks = (max_padded + 15) / 16;
+    int max_blocks = (max_padded + 15) / 16;
+    if (max_blocks < kDecodePairs) max_blocks = kDecodePairs;   // the in-kernel alignment numbers blocks by task
     size_t off = 0;
     auto take = [&](size_t bytes) {
         uint8_t *ptr = base ? base + off : nullptr;
@@ -568,7 +661,7 @@ static size_t carve(uint8_t *base, int tc, int E, int K, int inter, MoeWorkspace
     return off;
 }
 
-template <class T, bool FP8, int CB>
+template <class T, bool FP8, int CB, bool INLINE>
 static int launch_moe(const MoeArgs &a, int max_tasks, hipStream_t s) {
     // gate/up: one (gate, up) pair of row groups per wave for CB >= 2, two pairs for CB == 1
     constexpr int P = (CB == 1) ? 2 : 1;
@@ -579,29 +672,30 @@ static int launch_moe(const MoeArgs &a, int max_tasks, hipStream_t s) {
     while (g.WK * 64 > max_threads_for_tiles(2 * P * CB)) g.WK >>= 1;
     const int grid_x = groups_i / P;   // I % 128 == 0 so this is exact for P <= 8
     size_t lds1 = (size_t)g.WK * 2 * P * CB * 1024;
-    moe_gate_up_kernel<T, FP8, CB, P, U1><<<dim3(grid_x, max_tasks), g.WK * 64, lds1, s>>>(g);
+    moe_gate_up_kernel<T, FP8, CB, P, U1, INLINE><<<dim3(grid_x, max_tasks), g.WK * 64, lds1, s>>>(g);
     MLK_LAUNCH_CHECK();
 
     constexpr int R = 1;
-    constexpr int U2 = (CB >= 4) ? 3 : 4;
+    constexpr int U2 = (CB >= 4) ? 3 : (CB == 1 ? 8 : 4);
     MoeArgs d = a;
     d.WK = 16;
     while (d.WK > 1 && (d.WK * 64 > max_threads_for_tiles(R * CB) ||
-                        (size_t)d.WK * R * CB * 1024 + (size_t)a.T * 16 * R * 4 > 64 * 1024))
+                        (size_t)d.WK * R * CB * 1024 + (size_t)a.T * 16 * R * 4 + sizeof(DecodeTables) > 64 * 1024))
         d.WK >>= 1;
     size_t lds2 = (size_t)d.WK * R * CB * 1024 + (size_t)a.T * 16 * R * 4;
-    moe_down_kernel<T, FP8, CB, R, U2><<<a.H / 16 / R, d.WK * 64, lds2, s>>>(d);
+    moe_down_kernel<T, FP8, CB, R, U2, INLINE><<<a.H / 16 / R, d.WK * 64, lds2, s>>>(d);
     MLK_LAUNCH_CHECK();
     return MLK_OK;
 }
 
 template <class T, bool FP8>
-static int launch_moe_cb(const MoeArgs &a, int cb, int max_tasks, hipStream_t s) {
+static int launch_moe_cb(const MoeArgs &a, int cb, int max_tasks, bool inline_align, hipStream_t s) {
+    if (inline_align) return launch_moe<T, FP8, 1, true>(a, max_tasks, s);
     switch (cb) {
-        case 1: return launch_moe<T, FP8, 1>(a, max_tasks, s);
-        case 2: return launch_moe<T, FP8, 2>(a, max_tasks, s);
-        case 3: return launch_moe<T, FP8, 3>(a, max_tasks, s);
-        default: return launch_moe<T, FP8, 4>(a, max_tasks, s);
+        case 1: return launch_moe<T, FP8, 1, false>(a, max_tasks, s);
+        case 2: return launch_moe<T, FP8, 2, false>(a, max_tasks, s);
+        case 3: return launch_moe<T, FP8, 3, false>(a, max_tasks, s);
+        default: return launch_moe<T, FP8, 4, false>(a, max_tasks, s);
     }
 }
 
@@ -667,6 +761,7 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
     MLK_REQUIRE(topk >= 1 && topk <= kMaxTopK, "moe: topk must be in 1..32");
     MLK_REQUIRE(hidden > 0 && inter > 0 && hidden % 128 == 0 && inter % 128 == 0,
                 "moe: hidden and intermediate sizes must be multiples of 128");
+    MLK_REQUIRE(hidden <= kMaxScaleK && inter <= kMaxScaleK, "moe: hidden and intermediate sizes up to 32768");
     const bool fp8 = w_kind == MLK_FP8_E4M3;
     if (fp8) MLK_REQUIRE(x_kind == MLK_BF16, "moe: soft-FP8 weights need bf16 activations");
     else MLK_REQUIRE(w_kind == x_kind, "moe: weights and activations must have the same 16-bit type");
@@ -683,13 +778,18 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
         MoeWorkspace ws;
         carve((uint8_t *)workspace, tc, n_experts, topk, inter, &ws);
         const int max_padded = n_pairs + n_experts * 15;
-        const int max_blocks = (max_padded + 15) / 16;
+        int max_blocks = (max_padded + 15) / 16;
+        if (max_blocks < kDecodePairs) max_blocks = kDecodePairs;
         const int active = n_experts < n_pairs ? n_experts : n_pairs;
         const int max_tasks = active + n_pairs / (16 * cb);
-        moe_align_kernel<<<1, 1024, 0, s>>>(topk_ids + (size_t)t0 * topk, n_pairs, n_experts, experts_map, ws.sorted,
-                                            ws.cumsum, ws.padded, ws.experts_ids, max_blocks, ws.tasks, ws.n_tasks,
-                                            cb);
-        MLK_LAUNCH_CHECK();
+        // decode-sized batches align inside the GeMM kernels; larger ones run the alignment kernel
+        const bool inline_align = tc <= 16 && n_pairs <= kDecodePairs;
+        if (!inline_align) {
+            moe_align_kernel<<<1, 1024, 0, s>>>(topk_ids + (size_t)t0 * topk, n_pairs, n_experts, experts_map,
+                                                ws.sorted, ws.cumsum, ws.padded, ws.experts_ids, max_blocks, ws.tasks,
+                                                ws.n_tasks, cb);
+            MLK_LAUNCH_CHECK();
+        }
         MoeArgs a;
         a.W1 = (const uint8_t *)w1;
         a.W2 = (const uint8_t *)w2;
@@ -709,10 +809,13 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
         a.SB = max_blocks;
         a.n_pairs = n_pairs;
         a.WK = 1;
+        a.E = n_experts;
+        a.topk_ids = topk_ids + (size_t)t0 * topk;
+        a.experts_map = experts_map;
         int rc;
-        if (fp8) rc = launch_moe_cb<BF16, true>(a, cb, max_tasks, s);
-        else if (x_kind == MLK_F16) rc = launch_moe_cb<F16, false>(a, cb, max_tasks, s);
-        else rc = launch_moe_cb<BF16, false>(a, cb, max_tasks, s);
+        if (fp8) rc = launch_moe_cb<BF16, true>(a, cb, max_tasks, inline_align, s);
+        else if (x_kind == MLK_F16) rc = launch_moe_cb<F16, false>(a, cb, max_tasks, inline_align, s);
+        else rc = launch_moe_cb<BF16, false>(a, cb, max_tasks, inline_align, s);
         if (rc != MLK_OK) return rc;
     }
     return MLK_OK;

@@ -84,7 +84,7 @@ def test_gemv_soft_fp8_all_codes_exact(mlk):
     w[:, 5] = codes
     x = torch.zeros((1, k), dtype=torch.bfloat16)
     x[0, 5] = 1.0
-    for s in (1.0, 0.37, 1.0 / 448.0):
+    for s in (1.0, 0.37, 1.0 / 448.0, 0.5, 2.0 ** -7, 4.0):
         scale = torch.full((2, 1), s, dtype=torch.float32)
         y = mlk.gemv_layoutA(pack_a(w).cuda(), x.cuda(), scale_matrix=scale.cuda())
         want = softfp8.bf16_bits_to_f32(softfp8.dequant_bf16_bits(codes.numpy(), np.float32(s)))
