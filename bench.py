@@ -125,7 +125,10 @@ def main():
         scale = torch.ones((n // 128, k // 128), dtype=torch.float32, device=dev) if kind == 2 else None
         table = "layoutA_soft_fp8_gemm" if kind == 2 else ("layout_gemm" if native else "layoutA_gemm")
         kid, p1, p2, p3 = mlk.ops._gemm_guard(arg_selector.selector(table).get_args((n, m, k)), n)
-        p3 = 1
+        ws_ptr, ws_len = 0, 0
+        if p3 > 1:
+            ws = mlk.ops._workspace(dev, lib.mlk_gemm_workspace_bytes(m, n, p1, p3), lib.mlk_gemm_counter_bytes())
+            ws_ptr, ws_len = ws.data_ptr(), ws.numel()
         if native:
             b_in = mlk.layoutB(b)
             c = torch.empty((n // 32, m // 16, 4, 16, 8), dtype=DT[xk], device=dev)
@@ -139,7 +142,8 @@ def main():
                 st = torch.cuda.current_stream().cuda_stream
                 _lib.check(lib.mlk_gemm_layout_a(a.data_ptr(), b_in.data_ptr(), c.data_ptr(), m, n, k, kind, xk,
                                                  1 if native else 0, 1 if native else 0, 1.0, 0,
-                                                 0 if scale is None else scale.data_ptr(), kid, p1, p2, p3, 0, 0, st),
+                                                 0 if scale is None else scale.data_ptr(), kid, p1, p2, p3, ws_ptr, ws_len,
+                                                 st),
                            "gemm")
                 if native:
                     _lib.check(lib.mlk_re_layout_c(c.data_ptr(), c_rm.data_ptr(), m, n, st), "reLayoutC")
@@ -200,11 +204,28 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
+    def read_ceiling(steps):
+        """Pure streaming read of 256 MiB buffers (4 rotating copies) with the GeMV access pattern."""
+        nbytes = 256 << 20
+        bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(4)]
+        best = 0.0
+        for block, wgs in ((512, 2048), (1024, 1024), (256, 4096)):
+            def mk(b):
+                def call():
+                    _lib.check(lib.mlk_stream_read(b.data_ptr(), nbytes, block, wgs, 0,
+                                                   torch.cuda.current_stream().cuda_stream), "stream_read")
+                return call
+            us, _ = run_graph([mk(b) for b in bufs], steps, 5)
+            best = max(best, nbytes / us / 1e3)
+        return best
+
     # ------------------------------------------------------------ headline
     N, K_, M = 11008, 4096, 16
     head = gemm_case("C2 fp16 gemm_layoutA 11008x4096 M=16", N, K_, 0, M, args.steps, args.warmup)
     per_config = []
+    ceiling = None
     if not args.quick:
+        ceiling = round(read_ceiling(40), 1)
         short = max(20, min(args.steps, 100))
         per_config.append(gemv_case("C1 bf16 gemv 4096x4096", 4096, 4096, 1, short, 10))
         for m in (1, 8, 32, 64):
@@ -275,6 +296,9 @@ def main():
                    "algorithmic_bytes": head["bytes"]},
         "roofline": {"bound": "hbm", "achieved": round(head["gbps"], 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(head["frac"], 4), "traffic": traffic},
+        "hbm_read_ceiling": None if ceiling is None else {
+            "value": ceiling, "unit": "GB/s",
+            "what": "pure streaming read (mlk_stream_read, 256 MiB x 4 rotating buffers) measured in this run"},
         "cpu_baseline": cpu,
         "per_config": per_config,
     }

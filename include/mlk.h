@@ -78,6 +78,12 @@ int mlk_re_layout_c(const void *src, void *dst, int m, int n, void *stream);
  * covers the whole tensor (the reference skips partial 256x256 blocks). */
 int mlk_fp8_weight_repack(const void *src, void *dst, int64_t nbytes, void *stream);
 
+/* Measurement aid: read `nbytes` (a multiple of 1024) once with the GeMV kernels' access pattern
+ * and do nothing else; `workgroups` must divide nbytes/1024, `sink` is a device word that is never
+ * written in practice (may be NULL).  Used by bench.py to report the read bandwidth the memory
+ * system delivers to a pure streaming kernel next to the 8 TB/s peak.  No counterpart in the reference. */
+int mlk_stream_read(const void *src, int64_t nbytes, int block_dim_x, int workgroups, void *sink, void *stream);
+
 /* ---------------------------------------------------------------------- GeMV
  * y[M, N] = T(alpha * x[M, K] . A^T (+ bias[N])), 1 <= M <= 4, fp32 accumulate,
  * A in layout-A.  Replaces `gemv_layoutA` / `gemv_layoutA_wapper`,

@@ -329,7 +329,8 @@ static int launch(const GemmArgs &p, hipStream_t s) {
         const int tiles_total = q.K / 32;
         const int tiles_per = (tiles_total + q.SK - 1) / q.SK;
         const size_t win_bytes = (size_t)2 * q.WK * CB * 68 * 16;
-        if (g_tunable[1] && q.WK >= 2 && tiles_total % q.SK == 0 && tiles_per % q.WK == 0 && win_bytes <= 48 * 1024) {
+        // (measured: staging pays only from three token blocks up; below that the direct gather wins)
+        if (g_tunable[1] && CB >= 3 && q.WK >= 2 && tiles_total % q.SK == 0 && tiles_per % q.WK == 0 && win_bytes <= 48 * 1024) {
             constexpr int US = (R * CB >= 8) ? 2 : 4;
             if (win_bytes > lds) lds = win_bytes;
             gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, US, true><<<grid, q.WK * 64, lds, s>>>(q);

@@ -72,6 +72,48 @@ __global__ void __launch_bounds__(256) fp8_repack_kernel(const uint32_t *__restr
     }
 }
 
+// Pure streaming read with the access pattern of the GeMV kernels (1 KiB tiles, 16 bytes per
+// lane, non-temporal, U loads in flight per wave): measures what the memory system delivers to
+// a kernel that does nothing else.  The xor of everything read is compared with a value the
+// data never produces, so the loads cannot be optimised away and nothing is written.
+template <int U>
+__global__ void __launch_bounds__(1024) stream_read_kernel(const u32x4 *__restrict__ src, int64_t tiles_per_wg,
+                                                           uint32_t *__restrict__ sink) {
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int waves = blockDim.x >> 6;
+    const u32x4 *base = src + (size_t)blockIdx.x * tiles_per_wg * 64 + lane;
+    const int nt = wave < tiles_per_wg ? (int)((tiles_per_wg - wave + waves - 1) / waves) : 0;
+    u32x4 acc = {0u, 0u, 0u, 0u};
+    u32x4 buf[U];
+    auto ld = [&](int j) { return ld_stream_u32x4(base + (size_t)(wave + (int64_t)j * waves) * 64); };
+    if (nt >= U) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) buf[u] = ld(u);
+        int i = 0;
+        for (; i + 2 * U <= nt; i += U) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                acc ^= buf[u];
+                buf[u] = ld(i + U + u);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        const int rem = nt - i - U;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            acc ^= buf[u];
+            if (u < rem) buf[u] = ld(i + U + u);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < rem) acc ^= buf[u];
+    } else {
+        for (int j = 0; j < nt; ++j) acc ^= ld(j);
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x9e3779b9u && sink) sink[threadIdx.x & 63] = acc[0];
+}
+
 static inline int grid_for(int64_t total) {
     int64_t blocks = (total + 255) / 256;
     const int64_t cap = 256 * 32;  // 32 workgroups per CU is plenty for a copy
@@ -138,6 +180,21 @@ int mlk_re_layout_c(const void *src, void *dst, int m, int n, void *stream) {
     MLK_REQUIRE(src && dst, "reLayoutC: null pointer");
     layout_b_kernel<false><<<grid_for(total), 256, 0, (hipStream_t)stream>>>((const uint4 *)src, (uint4 *)dst, total,
                                                                             m / 16, n / 8);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+int mlk_stream_read(const void *src, int64_t nbytes, int block_dim_x, int workgroups, void *sink, void *stream) {
+    MLK_REQUIRE(nbytes >= 0 && nbytes % 1024 == 0, "stream_read: byte count must be a multiple of 1024");
+    MLK_REQUIRE(block_dim_x >= 64 && block_dim_x <= 1024 && block_dim_x % 64 == 0,
+                "stream_read: threads per workgroup must be a multiple of 64 in 64..1024");
+    MLK_REQUIRE(workgroups >= 1, "stream_read: at least one workgroup");
+    if (nbytes == 0) return MLK_OK;
+    MLK_REQUIRE(src, "stream_read: null pointer");
+    int64_t tiles = nbytes / 1024;
+    MLK_REQUIRE(tiles % workgroups == 0, "stream_read: the workgroup count must divide the number of 1 KiB tiles");
+    stream_read_kernel<4><<<workgroups, block_dim_x, 0, (hipStream_t)stream>>>((const u32x4 *)src, tiles / workgroups,
+                                                                              (uint32_t *)sink);
     MLK_LAUNCH_CHECK();
     return MLK_OK;
 }

@@ -32,12 +32,12 @@ DEFAULT_SHAPES = {
     "gemv_fp16": [(11008, 4096), (4096, 4096), (4096, 11008)],
     "gemv_bf16": [(4096, 4096), (28672, 8192), (8192, 8192), (28672, 4096), (4096, 14336)],
     "gemv_soft_fp8": [(28672, 8192), (4096, 4096), (8192, 8192)],
-    "layoutA_gemm": [(11008, 4096)],
+    "layoutA_gemm": [(11008, 4096), (4096, 4096), (4096, 11008)],
     "layoutA_soft_fp8_gemm": [(28672, 8192)],
-    "continuous_gemm": [(8192, 8192)],
-    "layout_gemm": [(8192, 8192)],
+    "continuous_gemm": [(8192, 8192), (11008, 4096)],
+    "layout_gemm": [(8192, 8192), (11008, 4096)],
 }
-DEFAULT_TOKENS = {"layoutA_gemm": [1, 8, 16, 32, 64], "layoutA_soft_fp8_gemm": [1, 4, 16],
+DEFAULT_TOKENS = {"layoutA_gemm": [1, 8, 16, 32, 48, 64], "layoutA_soft_fp8_gemm": [1, 4, 16, 32, 64],
                   "continuous_gemm": [16, 32, 64], "layout_gemm": [16, 32, 64]}
 MALL_BYTES = 256 << 20
 
@@ -137,16 +137,16 @@ def scan_gemm(table, shapes, tokens, iters):
             for p1 in (1, 2, 4):
                 if (n // 16) % p1:
                     continue
-                for p2 in (1, 2, 4, 8, 16):
+                for p2, p3 in [(w, sk) for w in (1, 2, 4, 8, 16) for sk in ((1, 2, 4) if n <= 8192 else (1,))]:
                     def call(a):
                         if mode == "rowmajor":
-                            return lambda: ops.gemm_layoutA_wapper(a, b_in, n, m, k, 1, 0, p1, p2, 1, 1, None)
+                            return lambda: ops.gemm_layoutA_wapper(a, b_in, n, m, k, 1, 0, p1, p2, p3, 1, None)
                         if mode == "fp8":
-                            return lambda: ops.gemm_layoutA_soft_fp8_wapper(a, scale, b_in, n, m, k, 1, 0, p1, p2, 1, 1,
+                            return lambda: ops.gemm_layoutA_soft_fp8_wapper(a, scale, b_in, n, m, k, 1, 0, p1, p2, p3, 1,
                                                                             None)
                         if mode == "continuous":
-                            return lambda: ops.gemm_layoutAB_ContinuousC_wapper(a, b_in, n, m, k, 1, 0, p1, p2, 1, 1, None)
-                        return lambda: ops.gemm_layoutABC_wapper(a, b_in, n, m, k, 1, 0, p1, p2, 1, 1, None)
+                            return lambda: ops.gemm_layoutAB_ContinuousC_wapper(a, b_in, n, m, k, 1, 0, p1, p2, p3, 1, None)
+                        return lambda: ops.gemm_layoutABC_wapper(a, b_in, n, m, k, 1, 0, p1, p2, p3, 1, None)
                     got = call(packed[0])()
                     if mode == "native":
                         got = ops.reLayoutC(got)
@@ -154,7 +154,7 @@ def scan_gemm(table, shapes, tokens, iters):
                         continue
                     us = _time_graph([call(a) for a in packed], iters)
                     if best is None or us < best[0]:
-                        best = (us, 1, p1, p2, 1)
+                        best = (us, 1, p1, p2, p3)
             print("%s %dx%d M=%d -> %s" % (table, n, k, m, best), file=sys.stderr)
             rows.append("%d,%d,%d,%d,%d,%d,%d" % (n, m, k, best[1], best[2], best[3], best[4]))
         del plain, packed
