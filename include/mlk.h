@@ -50,6 +50,9 @@ const char *mlk_last_error(void);
  * id 0 = rotate the k-tile visiting order of the narrow GeMM per row tile (default 1).
  * No counterpart in the reference. */
 void mlk_set_tunable(int id, int value);
+/* Experiment switch: use (1, default) or avoid (0) the row-shared kernels of the fused MoE for
+ * more than 16 tokens.  No counterpart in the reference. */
+void mlk_moe_set_tile_path(int on);
 
 /* ------------------------------------------------------------------ relayout
  * Pure permutations of 16-byte (16-bit elements) or 8-byte (fp8) granules;

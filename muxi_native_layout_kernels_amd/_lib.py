@@ -18,6 +18,7 @@ SIGNATURES = {
     "mlk_version": (c_int, []),
     "mlk_last_error": (ctypes.c_char_p, []),
     "mlk_set_tunable": (None, [c_int, c_int]),
+    "mlk_moe_set_tile_path": (None, [c_int]),
     "mlk_pack_layout_a": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
     "mlk_unpack_layout_a": (c_int, [c_void_p, c_void_p, c_int64, c_int, c_int, c_int, c_void_p]),
     "mlk_layout_b": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),

@@ -18,7 +18,9 @@ What the columns select on gfx950 (the rows are produced by the scripts in
                 KernelParam1 row groups (16 rows) per workgroup
                 KernelParam2 16-byte loads kept in flight per wave
   GEMM tables   m,n,k -> kernelId, kernelParam1, kernelParam2, kernelParam3
-                kernelId     1 = wave-tiled MFMA kernel
+                kernelId     1 = wave-tiled MFMA kernel (waves of a workgroup split K)
+                             2 = row-shared tile kernel (4 waves share the activations of
+                                 each k window through LDS; kernelParam2 is not used)
                 kernelParam1 row groups per wave (1, 2, 4)
                 kernelParam2 waves per workgroup splitting K (1..16)
                 kernelParam3 K splits across workgroups

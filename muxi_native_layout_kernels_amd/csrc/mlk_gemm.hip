@@ -19,7 +19,7 @@
 // layout-C -> row-major permutation equals the row-major output bit for bit.
 //
 // Algorithmic traffic per call: N*K*sizeof(W) (+ scales) + M*K*2 + M*N*2 bytes.
-#include "mlk_gemm_tile.cuh"
+#include "mlk_tile.cuh"
 
 namespace mlk {
 
@@ -316,6 +316,123 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel
     }
 }
 
+// Kernel 2: row-shared tile kernel (see mlk_tile.cuh).  Four waves per workgroup, R row groups
+// per wave, activations of every k window staged once per workgroup in LDS; K is split across
+// workgroups only (SK), folded by the last workgroup to arrive with agent-coherent loads.
+template <class T, bool FP8, int CB, int R, int BMODE, int CMODE>
+__global__ void __launch_bounds__(256) gemm_tile_kernel(GemmArgs p) {
+    extern __shared__ u32x4 tile_win[];
+    __shared__ int s_last;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = lane >> 4, r16 = lane & 15;
+    const int sk = blockIdx.x % p.SK;
+    const int rt = blockIdx.x / p.SK;
+    const int rg0 = (rt * kTileWaves + wave) * R;
+    const int tiles_total = p.K >> 5;
+    const int tiles_per = tiles_total / p.SK;          // host: a whole number of windows
+    const int tbeg = sk * tiles_per, tend = tbeg + tiles_per;
+    const int mb_total = (p.M_total + 15) >> 4;
+    const int scale_cols = (p.K + 127) >> 7;
+    constexpr int WBYTES = FP8 ? 1 : 2;
+
+    const uint8_t *abase[R];
+    ScaleRow srow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        abase[r] = p.A + (size_t)(rg0 + r) * p.K * 16 * WBYTES;
+        if (FP8)
+            srow[r] = load_scale_row(p.scale ? p.scale + (size_t)((rg0 + r) >> 3) * scale_cols : nullptr, scale_cols, lane);
+    }
+    TileBSource<CB> bs;
+    if (BMODE == MLK_B_NATIVE) {
+        bs.native_tile_stride = (size_t)mb_total * 512;
+        bs.row[0] = p.B + (size_t)p.cb0 * 512;
+    } else {
+        bs.native_tile_stride = 0;
+#pragma unroll
+        for (int i = 0; i < tile_granules_per_thread<CB>(); ++i) {
+            int block, token, colg;
+            tile_row_of<CB>(i, threadIdx.x, block, token, colg);
+            const int tok = min((p.cb0 + block) * 16 + token, p.M_total - 1);
+            bs.row[i] = p.B + (size_t)tok * p.K + colg * 8;
+        }
+    }
+    f32x4 acc[R][CB];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    TileLoop<T, FP8, CB, R>::run(acc, abase, srow, bs, tbeg, tend, tile_win, p.rotate ? rt : 0);
+
+    constexpr int NTILE = R * CB;
+    const int row_tiles = gridDim.x / p.SK;
+    auto epilogue = [&](int r, int cb, f32x4 v) {
+        const int n = (rg0 + r) * 16 + 4 * q;
+        const int tok = (p.cb0 + cb) * 16 + r16;
+        if (tok >= p.M_total) return;
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o[i] = p.alpha * v[i];
+            if (p.bias) o[i] += T::to_f32(p.bias[n + i]);
+        }
+        size_t off;
+        if (CMODE == MLK_C_NATIVE)
+            off = ((((size_t)(n >> 5) * mb_total + (tok >> 4)) * 4 + ((n & 31) >> 3)) * 16 + (tok & 15)) * 8 + (n & 7);
+        else
+            off = (size_t)tok * p.N + n;
+        store4<T>(p.C + off, o[0], o[1], o[2], o[3]);
+    };
+    if (p.SK == 1) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) epilogue(r, cb, acc[r][cb]);
+        return;
+    }
+    f32x4 *part = reinterpret_cast<f32x4 *>(p.partial);
+    auto part_at = [&](int s, int j) -> size_t {
+        return ((((size_t)s * row_tiles + rt) * kTileWaves + wave) * NTILE + j) * 64 + lane;
+    };
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) st_agent_f32x4(&part[part_at(sk, r * CB + cb)], acc[r][cb]);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int prev = __hip_atomic_fetch_add(&p.counters[rt], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (prev == p.SK - 1);
+        if (s_last) __hip_atomic_store(&p.counters[rt], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last) return;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            for (int s = 0; s < p.SK; ++s) v += ld_agent_f32x4(&part[part_at(s, r * CB + cb)]);
+            epilogue(r, cb, v);
+        }
+}
+
+// Can kernel 2 run this problem with these parameters?
+static bool tile_kernel_fits(const GemmArgs &p, int R) {
+    const int tiles_total = p.K / 32;
+    return (p.N / 16) % (kTileWaves * R) == 0 && p.SK >= 1 && tiles_total % (p.SK * kTileKW) == 0;  // CB <= 4 here
+}
+
+template <class T, bool FP8, int CB, int R, int BMODE, int CMODE>
+static int launch_tile(const GemmArgs &p, hipStream_t s) {
+    int row_tiles = (p.N / 16) / (kTileWaves * R);
+    gemm_tile_kernel<T, FP8, CB, R, BMODE, CMODE><<<row_tiles * p.SK, 256, tile_lds_bytes<CB>(), s>>>(p);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
 template <class T, bool FP8, int CB, int R, int BMODE, int CMODE>
 static int launch(const GemmArgs &p, hipStream_t s) {
     constexpr int U = (R * CB >= 8) ? 2 : ((R * CB >= 4) ? 3 : 4);
@@ -344,9 +461,11 @@ static int launch(const GemmArgs &p, hipStream_t s) {
 }
 
 template <class T, bool FP8, int BMODE, int CMODE>
-static int launch_rc(const GemmArgs &p, int R, int CB, hipStream_t s) {
-#define MLK_CASE(RR, CC) \
-    if (R == RR && CB == CC) return launch<T, FP8, CC, RR, BMODE, CMODE>(p, s);
+static int launch_rc(const GemmArgs &p, int kernel_id, int R, int CB, hipStream_t s) {
+#define MLK_CASE(RR, CC)                                                                        \
+    if (R == RR && CB == CC)                                                                    \
+        return (kernel_id == 2 && tile_kernel_fits(p, RR)) ? launch_tile<T, FP8, CC, RR, BMODE, CMODE>(p, s) \
+                                                          : launch<T, FP8, CC, RR, BMODE, CMODE>(p, s);
     MLK_CASE(1, 1) MLK_CASE(1, 2) MLK_CASE(1, 3) MLK_CASE(1, 4)
     MLK_CASE(2, 1) MLK_CASE(2, 2) MLK_CASE(2, 3) MLK_CASE(2, 4)
     MLK_CASE(4, 1) MLK_CASE(4, 2) MLK_CASE(4, 3) MLK_CASE(4, 4)
@@ -355,14 +474,14 @@ static int launch_rc(const GemmArgs &p, int R, int CB, hipStream_t s) {
 }
 
 template <class T, bool FP8>
-static int launch_modes(const GemmArgs &p, int b_mode, int c_mode, int R, int CB, hipStream_t s) {
+static int launch_modes(const GemmArgs &p, int kernel_id, int b_mode, int c_mode, int R, int CB, hipStream_t s) {
     if (b_mode == MLK_B_ROWMAJOR && c_mode == MLK_C_ROWMAJOR)
-        return launch_rc<T, FP8, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR>(p, R, CB, s);
+        return launch_rc<T, FP8, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR>(p, kernel_id, R, CB, s);
     if (!FP8) {
         if (b_mode == MLK_B_NATIVE && c_mode == MLK_C_ROWMAJOR)
-            return launch_rc<T, false, MLK_B_NATIVE, MLK_C_ROWMAJOR>(p, R, CB, s);
+            return launch_rc<T, false, MLK_B_NATIVE, MLK_C_ROWMAJOR>(p, kernel_id, R, CB, s);
         if (b_mode == MLK_B_NATIVE && c_mode == MLK_C_NATIVE)
-            return launch_rc<T, false, MLK_B_NATIVE, MLK_C_NATIVE>(p, R, CB, s);
+            return launch_rc<T, false, MLK_B_NATIVE, MLK_C_NATIVE>(p, kernel_id, R, CB, s);
     }
     return fail(MLK_ERR_INVALID, "gemm: unsupported operand placement");
 }
@@ -392,7 +511,7 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
     MLK_REQUIRE(m >= 0 && n >= 0 && k >= 0, "gemm: negative size");
     MLK_REQUIRE(n % 16 == 0, "gemm: N % 16 must be 0");
     MLK_REQUIRE(k % 32 == 0, "gemm: K % 32 must be 0");
-    MLK_REQUIRE(kernel_id == 1, "gemm: unknown kernel id");
+    MLK_REQUIRE(kernel_id == 1 || kernel_id == 2, "gemm: unknown kernel id");
     MLK_REQUIRE(p1 == 1 || p1 == 2 || p1 == 4, "gemm: row groups per wave (p1) must be 1, 2 or 4");
     MLK_REQUIRE((n / 16) % p1 == 0, "gemm: row groups per wave (p1) must divide N/16");
     MLK_REQUIRE(p2 == 1 || p2 == 2 || p2 == 4 || p2 == 8 || p2 == 16, "gemm: waves per workgroup (p2) must be 1, 2, 4, 8 or 16");
@@ -418,6 +537,7 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
     if (sk > 1) {
         MLK_REQUIRE(workspace != nullptr, "gemm: a K split across workgroups needs a workspace");
         MLK_REQUIRE((size_t)(n / 16 / p1) * sizeof(int) <= kCounterBytes, "gemm: too many row tiles for the counter region");
+        if (kernel_id == 2 && (k / 32) % (sk * kTileKW) != 0) sk = 1;   // kernel 2 splits K in whole windows only
         size_t need = kCounterBytes + (size_t)sk * (size_t)(n / 16) * cb_max * 1024;
         if (workspace_bytes < need) return fail(MLK_ERR_WORKSPACE, "gemm: workspace too small");
     }
@@ -446,9 +566,9 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
         g.cb0 = c0 / 16;
         int cb = (mm + 15) / 16;
         int rc;
-        if (fp8) rc = launch_modes<BF16, true>(g, b_mode, c_mode, p1, cb, s);
-        else if (x_kind == MLK_F16) rc = launch_modes<F16, false>(g, b_mode, c_mode, p1, cb, s);
-        else rc = launch_modes<BF16, false>(g, b_mode, c_mode, p1, cb, s);
+        if (fp8) rc = launch_modes<BF16, true>(g, kernel_id, b_mode, c_mode, p1, cb, s);
+        else if (x_kind == MLK_F16) rc = launch_modes<F16, false>(g, kernel_id, b_mode, c_mode, p1, cb, s);
+        else rc = launch_modes<BF16, false>(g, kernel_id, b_mode, c_mode, p1, cb, s);
         if (rc != MLK_OK) return rc;
     }
     return MLK_OK;

@@ -22,13 +22,25 @@
 // Algorithmic traffic per layer: active experts * 3*I*H*sizeof(W) (+ scales)
 // + 2*T*H*2 + T*E*2 bytes; the SiLU intermediate (T*K*I*2 bytes, written and
 // read once) stays in L2 / Infinity Cache for decode-sized T.
-#include "mlk_gemm_tile.cuh"
+#include "mlk_tile.cuh"
 
 namespace mlk {
 
 constexpr int kMaxExperts = 256;
 constexpr int kMaxTopK = 32;
 constexpr int kMoeChunk = 256;     // tokens per expert-compute pass
+static int g_moe_tile = 1;         // experiment switch: row-shared kernels for tasks of more than one token block
+static inline bool moe_tile_path() { return g_moe_tile != 0; }
+// Token blocks per task: as many as the largest possible expert load needs, at most 8 with the
+// row-shared kernels (4 without); 5 and 7 round up to the next instantiated width.
+static inline int moe_blocks_per_task(int tokens) {
+    int cb = (tokens + 15) / 16;
+    const int cap = moe_tile_path() ? 8 : 4;
+    if (cb > cap) cb = cap;
+    if (cb == 5) cb = 6;
+    if (cb == 7) cb = 8;
+    return cb;
+}
 
 // ------------------------------------------------------------------ router
 template <class T>
@@ -628,17 +640,156 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
     }
 }
 
+// ------------------------------------------------ row-shared variants (more than 16 tokens)
+// For tasks of two to four token blocks the four waves of a workgroup share the activation
+// windows through LDS (mlk_tile.cuh) instead of gathering them per wave.
+
+// gate/up: each wave owns P (gate, up) pairs of row groups, grid (I/(64 P), tasks)
+template <class T, bool FP8, int CB, int P>
+__global__ void __launch_bounds__(256) moe_gate_up_tile_kernel(MoeArgs p) {
+    extern __shared__ u32x4 tile_win[];
+    const int task = blockIdx.y;
+    if (task >= p.n_tasks[0]) return;
+    const MoeTask tk = p.tasks[task];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = lane >> 4, r16 = lane & 15;
+    const int g0 = (blockIdx.x * kTileWaves + wave) * P;   // first row group inside the gate (and the up) half
+    constexpr int WB = FP8 ? 1 : 2;
+    constexpr int R = 2 * P;                               // streams: gate, up, gate, up ...
+    const int groups_i = p.I >> 4;
+    const size_t slab = (size_t)2 * p.I * p.H * WB;
+    const int scale_cols = p.H >> 7;
+
+    const uint8_t *abase[R];
+    ScaleRow srow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int rg = (r & 1) * groups_i + g0 + (r >> 1);
+        abase[r] = p.W1 + (size_t)tk.expert * slab + (size_t)rg * p.H * 16 * WB;
+        if (FP8)
+            srow[r] = load_scale_row(
+                p.S1 ? p.S1 + ((size_t)tk.expert * (2 * p.I >> 7) + (rg >> 3)) * scale_cols : nullptr, scale_cols, lane);
+    }
+    TileBSource<CB> bs;
+    bs.native_tile_stride = 0;
+#pragma unroll
+    for (int i = 0; i < tile_granules_per_thread<CB>(); ++i) {
+        int block, token, colg;
+        tile_row_of<CB>(i, threadIdx.x, block, token, colg);
+        int id = p.n_pairs;
+        if (block < tk.nblocks) id = p.sorted[(tk.block0 + block) * 16 + token];
+        bs.row[i] = p.X + (size_t)(id < p.n_pairs ? id / p.K : 0) * p.H + colg * 8;
+    }
+    f32x4 acc[R][CB];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    TileLoop<T, FP8, CB, R>::run(acc, abase, srow, bs, 0, p.H >> 5, tile_win, blockIdx.x + 7 * task);
+#pragma unroll
+    for (int pr = 0; pr < P; ++pr)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            if (cb >= tk.nblocks) continue;
+            float h[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                h[i] = acc[2 * pr][cb][i] / (1.f + __expf(-acc[2 * pr][cb][i])) * acc[2 * pr + 1][cb][i];
+            const int n = (g0 + pr) * 16 + 4 * q;
+            const size_t off =
+                ((((size_t)(n >> 5) * p.SB + (tk.block0 + cb)) * 4 + ((n & 31) >> 3)) * 16 + r16) * 8 + (n & 7);
+            store4<T>(p.Hbuf + off, h[0], h[1], h[2], h[3]);
+        }
+}
+
+// down: each wave owns R row groups of the output, grid (H/(64 R), tasks, K slices); the
+// routing-weighted partial products go to an fp32 buffer indexed by (pair, K slice), summed per
+// token in a fixed order by moe_combine_kernel
+template <class T, bool FP8, int CB, int R>
+__global__ void __launch_bounds__(256) moe_down_tile_kernel(MoeArgs p, float *__restrict__ O) {
+    extern __shared__ u32x4 tile_win[];
+    const int task = blockIdx.y;
+    if (task >= p.n_tasks[0]) return;
+    const MoeTask tk = p.tasks[task];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = lane >> 4, r16 = lane & 15;
+    const int rg0 = (blockIdx.x * kTileWaves + wave) * R;
+    constexpr int WB = FP8 ? 1 : 2;
+    const size_t slab = (size_t)p.H * p.I * WB;
+    const int scale_cols = p.I >> 7;
+
+    const uint8_t *abase[R];
+    ScaleRow srow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        abase[r] = p.W2 + (size_t)tk.expert * slab + (size_t)(rg0 + r) * p.I * 16 * WB;
+        if (FP8)
+            srow[r] = load_scale_row(
+                p.S2 ? p.S2 + ((size_t)tk.expert * (p.H >> 7) + ((rg0 + r) >> 3)) * scale_cols : nullptr, scale_cols, lane);
+    }
+    TileBSource<CB> bs;
+    bs.native_tile_stride = (size_t)p.SB * 512;
+    bs.row[0] = p.Hbuf + (size_t)tk.block0 * 512;          // CB consecutive blocks; those past the task are never used
+    f32x4 acc[R][CB];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    const int tiles_per = (p.I >> 5) / gridDim.z;          // host: a whole number of windows
+    TileLoop<T, FP8, CB, R>::run(acc, abase, srow, bs, blockIdx.z * tiles_per, (blockIdx.z + 1) * tiles_per, tile_win,
+                                 blockIdx.x + 7 * task);
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        if (cb >= tk.nblocks) continue;
+        const int id = p.sorted[(tk.block0 + cb) * 16 + r16];
+        if (id >= p.n_pairs) continue;
+        const float wt = T::to_f32(p.wts[id]);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            f32x4 v = acc[r][cb];
+            v *= wt;
+            *reinterpret_cast<f32x4 *>(O + ((size_t)id * gridDim.z + blockIdx.z) * p.H + (rg0 + r) * 16 + 4 * q) = v;
+        }
+    }
+}
+
+// y[t] = T(sum over the token's routed pairs, in pick order, of the weighted products)
+template <class T>
+__global__ void __launch_bounds__(256) moe_combine_kernel(const float *__restrict__ O, uint16_t *__restrict__ Y,
+                                                          const int32_t *__restrict__ topk_ids,
+                                                          const int32_t *__restrict__ experts_map, int K, int H,
+                                                          int E, int SKD) {
+    const int tok = blockIdx.x;
+    for (int n = threadIdx.x * 4; n < H; n += blockDim.x * 4) {
+        f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+        for (int k = 0; k < K; ++k) {
+            int e = topk_ids[tok * K + k];
+            if (experts_map) e = experts_map[e];
+            if (e < 0 || e >= E) continue;
+            f32x4 pair = {0.f, 0.f, 0.f, 0.f};
+            for (int sk = 0; sk < SKD; ++sk)
+                pair += *reinterpret_cast<const f32x4 *>(O + ((size_t)(tok * K + k) * SKD + sk) * H + n);
+            sum += pair;
+        }
+        store4<T>(Y + (size_t)tok * H + n, sum[0], sum[1], sum[2], sum[3]);
+    }
+}
+
 // ----------------------------------------------------------- host-side glue
 struct MoeWorkspace {
     MoeTask *tasks;
     int32_t *n_tasks;
     int32_t *sorted, *cumsum, *padded, *experts_ids;
     uint16_t *hbuf;
+    float *obuf;
+    int sb;          // token blocks the intermediate is dimensioned for
 };
 
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
-static size_t carve(uint8_t *base, int tc, int E, int K, int inter, MoeWorkspace *ws) {
+static size_t carve(uint8_t *base, int tc, int E, int K, int hidden, int inter, MoeWorkspace *ws) {
     const int n_pairs = tc * K;
     const int max_padded = n_pairs + E * 15;
     int max_blocks = (max_padded + 15) / 16;
@@ -656,7 +807,10 @@ static size_t carve(uint8_t *base, int tc, int E, int K, int inter, MoeWorkspace
     w.cumsum = (int32_t *)take(sizeof(int32_t) * (size_t)(E + 1));
     w.padded = (int32_t *)take(sizeof(int32_t));
     w.experts_ids = (int32_t *)take(sizeof(int32_t) * (size_t)max_blocks);
-    w.hbuf = (uint16_t *)take((size_t)inter * max_blocks * 16 * 2);
+    // seven spare blocks: the row-shared down kernel always fetches CB <= 8 consecutive blocks
+    w.sb = max_blocks + 7;
+    w.hbuf = (uint16_t *)take((size_t)inter * w.sb * 16 * 2);
+    w.obuf = (float *)take(tc > 16 ? (size_t)n_pairs * 8 * hidden * sizeof(float) : 0);   // 8 = kMoeMaxKSlices
     if (ws) *ws = w;
     return off;
 }
@@ -688,20 +842,55 @@ static int launch_moe(const MoeArgs &a, int max_tasks, hipStream_t s) {
     return MLK_OK;
 }
 
+constexpr int kMoeMaxKSlices = 8;  // K slices of the row-shared down projection (sizes its fp32 buffer)
+
+template <class T, bool FP8, int CB>
+static int launch_moe_tile(const MoeArgs &a, int max_tasks, float *obuf, hipStream_t s) {
+    // gate/up: two pairs of row groups per wave from five token blocks up (halves the activation re-reads)
+    constexpr int P = CB > 4 ? 2 : 1;
+    moe_gate_up_tile_kernel<T, FP8, CB, P>
+        <<<dim3(a.I / 16 / kTileWaves / P, max_tasks), 256, tile_lds_bytes<CB>(), s>>>(a);
+    MLK_LAUNCH_CHECK();
+    // down: R row groups per wave; the few output rows (H/16 row groups) are spread over enough
+    // workgroups by slicing K, each slice a whole number of windows
+    constexpr int R = CB > 4 ? 4 : 2;
+    const int groups_h = a.H / 16;
+    const int windows = (a.I / 32) / tile_kw<CB>();
+    if (groups_h % (R * kTileWaves) == 0) {
+        const int row_tiles = groups_h / (R * kTileWaves);
+        int skd = 1;
+        while (skd < kMoeMaxKSlices && row_tiles * max_tasks * skd < 512 && windows % (skd * 2) == 0) skd *= 2;
+        moe_down_tile_kernel<T, FP8, CB, R><<<dim3(row_tiles, max_tasks, skd), 256, tile_lds_bytes<CB>(), s>>>(a, obuf);
+        MLK_LAUNCH_CHECK();
+        moe_combine_kernel<T><<<a.T, 256, 0, s>>>(obuf, a.Y, a.topk_ids, a.experts_map, a.K, a.H, a.E, skd);
+    } else {
+        moe_down_tile_kernel<T, FP8, CB, 1><<<dim3(groups_h / kTileWaves, max_tasks, 1), 256, tile_lds_bytes<CB>(), s>>>(a, obuf);
+        MLK_LAUNCH_CHECK();
+        moe_combine_kernel<T><<<a.T, 256, 0, s>>>(obuf, a.Y, a.topk_ids, a.experts_map, a.K, a.H, a.E, 1);
+    }
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
 template <class T, bool FP8>
-static int launch_moe_cb(const MoeArgs &a, int cb, int max_tasks, bool inline_align, hipStream_t s) {
+static int launch_moe_cb(const MoeArgs &a, int cb, int max_tasks, bool inline_align, float *obuf, hipStream_t s) {
     if (inline_align) return launch_moe<T, FP8, 1, true>(a, max_tasks, s);
+    const bool tile = moe_tile_path();
     switch (cb) {
         case 1: return launch_moe<T, FP8, 1, false>(a, max_tasks, s);
-        case 2: return launch_moe<T, FP8, 2, false>(a, max_tasks, s);
-        case 3: return launch_moe<T, FP8, 3, false>(a, max_tasks, s);
-        default: return launch_moe<T, FP8, 4, false>(a, max_tasks, s);
+        case 2: return tile ? launch_moe_tile<T, FP8, 2>(a, max_tasks, obuf, s) : launch_moe<T, FP8, 2, false>(a, max_tasks, s);
+        case 3: return tile ? launch_moe_tile<T, FP8, 3>(a, max_tasks, obuf, s) : launch_moe<T, FP8, 3, false>(a, max_tasks, s);
+        case 4: return tile ? launch_moe_tile<T, FP8, 4>(a, max_tasks, obuf, s) : launch_moe<T, FP8, 4, false>(a, max_tasks, s);
+        case 6: return launch_moe_tile<T, FP8, 6>(a, max_tasks, obuf, s);
+        default: return launch_moe_tile<T, FP8, 8>(a, max_tasks, obuf, s);
     }
 }
 
 }  // namespace mlk
 
 using namespace mlk;
+
+extern "C" void mlk_moe_set_tile_path(int on) { g_moe_tile = on; }
 
 extern "C" int mlk_fused_routing_gate(const void *logits, int x_kind, int score_fun, int n_tokens, int n_experts,
                                       int n_groups, int topk_groups, int topk, const void *bias, int renormalize,
@@ -745,9 +934,8 @@ extern "C" int mlk_moe_align_tokens(const int32_t *topk_ids, int n_pairs, int n_
 }
 
 extern "C" size_t mlk_moe_workspace_bytes(int n_tokens, int n_experts, int topk, int hidden, int inter) {
-    (void)hidden;
     int tc = n_tokens < kMoeChunk ? n_tokens : kMoeChunk;
-    return carve(nullptr, tc, n_experts, topk, inter, nullptr);
+    return carve(nullptr, tc, n_experts, topk, hidden, inter, nullptr);
 }
 
 extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const void *x, int n_tokens, int n_experts,
@@ -774,9 +962,9 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
     for (int t0 = 0; t0 < n_tokens; t0 += kMoeChunk) {
         const int tc = n_tokens - t0 < kMoeChunk ? n_tokens - t0 : kMoeChunk;
         const int n_pairs = tc * topk;
-        const int cb = (tc + 15) / 16 < 4 ? (tc + 15) / 16 : 4;   // an expert sees at most tc tokens
+        const int cb = moe_blocks_per_task(tc);                  // an expert sees at most tc tokens
         MoeWorkspace ws;
-        carve((uint8_t *)workspace, tc, n_experts, topk, inter, &ws);
+        carve((uint8_t *)workspace, tc, n_experts, topk, hidden, inter, &ws);
         const int max_padded = n_pairs + n_experts * 15;
         int max_blocks = (max_padded + 15) / 16;
         if (max_blocks < kDecodePairs) max_blocks = kDecodePairs;
@@ -806,16 +994,16 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
         a.K = topk;
         a.H = hidden;
         a.I = inter;
-        a.SB = max_blocks;
+        a.SB = ws.sb;
         a.n_pairs = n_pairs;
         a.WK = 1;
         a.E = n_experts;
         a.topk_ids = topk_ids + (size_t)t0 * topk;
         a.experts_map = experts_map;
         int rc;
-        if (fp8) rc = launch_moe_cb<BF16, true>(a, cb, max_tasks, inline_align, s);
-        else if (x_kind == MLK_F16) rc = launch_moe_cb<F16, false>(a, cb, max_tasks, inline_align, s);
-        else rc = launch_moe_cb<BF16, false>(a, cb, max_tasks, inline_align, s);
+        if (fp8) rc = launch_moe_cb<BF16, true>(a, cb, max_tasks, inline_align, ws.obuf, s);
+        else if (x_kind == MLK_F16) rc = launch_moe_cb<F16, false>(a, cb, max_tasks, inline_align, ws.obuf, s);
+        else rc = launch_moe_cb<BF16, false>(a, cb, max_tasks, inline_align, ws.obuf, s);
         if (rc != MLK_OK) return rc;
     }
     return MLK_OK;

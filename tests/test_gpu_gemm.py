@@ -49,6 +49,42 @@ def test_gemm_launch_parameters(mlk, p1, p2, p3, m):
     assert torch.equal(c, c2), "K split across workgroups must be deterministic and leave its counters clean"
 
 
+@pytest.mark.parametrize("p1,p3", [(1, 1), (2, 1), (4, 1), (1, 2), (2, 4), (4, 8)])
+@pytest.mark.parametrize("m", [16, 33, 48, 64, 100])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gemm_tile_kernel(mlk, p1, p3, m, dtype):
+    """kernelId 2: row-shared tile kernel, row-major and native operands, K split across workgroups."""
+    n, k = 1024, 2048
+    w = randn((n, k), dtype, 0.02, 13)
+    b = randn((m, k), dtype, 1.0, 14)
+    bias = randn((1, n), dtype, 1.0, 15)
+    a = pack_a(w).cuda()
+    want = ogemm.linear_expected(w, b, 1.25, bias)
+    c = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=1.25, kernelParam1=p1, kernelParam2=1, kernelParam3=p3,
+                                kernelId=2, bias=bias.cuda())
+    assert_close(c, want, RTOL, ATOL, "tile kernel")
+    assert torch.equal(c, mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=1.25, kernelParam1=p1, kernelParam2=1,
+                                                  kernelParam3=p3, kernelId=2, bias=bias.cuda()))
+    if m % 16 == 0:
+        b_nat = mlk.layoutB(b.cuda())
+        c_rm = mlk.gemm_layoutAB_ContinuousC_wapper(a, b_nat, n, m, k, alpha=1.25, kernelParam1=p1, kernelParam3=p3,
+                                                    kernelId=2, bias=bias.cuda())
+        c_nat = mlk.gemm_layoutABC_wapper(a, b_nat, n, m, k, alpha=1.25, kernelParam1=p1, kernelParam3=p3, kernelId=2,
+                                          bias=bias.cuda())
+        assert torch.equal(c_rm, c) and torch.equal(mlk.reLayoutC(c_nat), c)
+
+
+def test_gemm_tile_kernel_soft_fp8(mlk):
+    n, k, m = 1024, 2048, 40
+    codes = fp8_codes((n, k), 21)
+    b = randn((m, k), torch.bfloat16, 1.0, 22)
+    g = torch.Generator().manual_seed(23)
+    scale = (torch.rand((n // 128, k // 128), generator=g) * 0.02 + 0.001).float()
+    c = mlk.gemm_layoutA_soft_fp8_wapper(pack_a(codes).cuda(), scale.cuda(), b.cuda(), n, m, k, kernelParam1=2,
+                                         kernelParam3=2, kernelId=2)
+    assert_close(c, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), b), RTOL, ATOL, "tile fp8")
+
+
 def test_gemm_special_cases(mlk):
     n = k = 256
     eye = torch.eye(n, dtype=torch.float16)

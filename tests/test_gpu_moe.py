@@ -144,7 +144,7 @@ def _moe_case(mlk, T, E, K, H, I, dtype, seed, score="softmax", fp8=False, group
     return y
 
 
-@pytest.mark.parametrize("T", [1, 2, 16, 17, 64, 100, 256, 300])
+@pytest.mark.parametrize("T", [1, 2, 16, 17, 40, 64, 70, 90, 100, 128, 256, 300])
 def test_fused_moe_small_shape(mlk, T):
     _moe_case(mlk, T, 8, 2, 256, 384, torch.bfloat16, 100 + T)
 
@@ -156,7 +156,7 @@ def test_fused_moe_dtypes_and_determinism(mlk, dtype):
     assert torch.equal(y1, y2)
 
 
-@pytest.mark.parametrize("T", [1, 16, 70])
+@pytest.mark.parametrize("T", [1, 16, 70, 130])
 def test_fused_moe_soft_fp8(mlk, T):
     _moe_case(mlk, T, 8, 2, 256, 384, torch.bfloat16, 300 + T, fp8=True)
 
