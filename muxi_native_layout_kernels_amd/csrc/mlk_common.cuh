@@ -128,9 +128,14 @@ __device__ __forceinline__ ScaleRow load_scale_row(const float *row, int cols, i
     return s;
 }
 __device__ __forceinline__ float scale_at(const ScaleRow &s, int kblock /* wave-uniform */) {
-    const int hi = kblock >> 6;
-    float x = hi == 0 ? s.v[0] : (hi == 1 ? s.v[1] : (hi == 2 ? s.v[2] : s.v[3]));
-    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(x), kblock & 63));
+    // four v_readlane and scalar selects: no branch, no vector select
+    const int l = kblock & 63, hi = kblock >> 6;
+    const int a0 = __builtin_amdgcn_readlane(__float_as_int(s.v[0]), l);
+    const int a1 = __builtin_amdgcn_readlane(__float_as_int(s.v[1]), l);
+    const int a2 = __builtin_amdgcn_readlane(__float_as_int(s.v[2]), l);
+    const int a3 = __builtin_amdgcn_readlane(__float_as_int(s.v[3]), l);
+    const int lo = (hi & 1) ? a1 : a0, up = (hi & 1) ? a3 : a2;
+    return __int_as_float((hi & 2) ? up : lo);
 }
 
 // 64-lane xor shuffle of an fp32 through the LDS crossbar (no LDS memory used).

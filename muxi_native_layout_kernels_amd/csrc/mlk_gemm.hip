@@ -98,20 +98,20 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel
 
     WeightFrag<FP8> wf[U][R];
     u32x4 bf[U][CB];
-    float sc[U][R];
+    float sc[U];        // one block scale per k tile: the R row groups of a wave share a 128-row block
     auto issue = [&](int slot, int kt) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
-            if (FP8) sc[slot][r] = scale_at(srow, kt >> 2);
-        }
+        for (int r = 0; r < R; ++r) wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
+        if (FP8) sc[slot] = scale_at(srow, kt >> 2);
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * bstep);
     };
     auto consume = [&](int slot) {
         u32x4 a[R], b[CB];
+        float sv[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) a[r] = weight_operand<FP8>(wf[slot][r], FP8 ? sc[slot][r] : 1.f);
+        for (int r = 0; r < R; ++r) sv[r] = FP8 ? sc[slot] : 1.f;
+        weight_operands<FP8, R>(a, wf[slot], sv);
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) b[cb] = bf[slot][cb];
 #pragma unroll
@@ -160,10 +160,8 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel
         auto issue_a = [&](int slot) {
             const int kt = tbeg + advance(w_issue) * p.WK + wave;
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
-                if (FP8) sc[slot][r] = scale_at(srow, kt >> 2);
-            }
+            for (int r = 0; r < R; ++r) wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
+            if (FP8) sc[slot] = scale_at(srow, kt >> 2);
         };
         auto step = [&](int slot, int buf, bool do_stage, bool do_issue) {
             if (do_stage) stage_load();
@@ -345,6 +343,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(GemmArgs p) {
             srow[r] = load_scale_row(p.scale ? p.scale + (size_t)((rg0 + r) >> 3) * scale_cols : nullptr, scale_cols, lane);
     }
     TileBSource<CB> bs;
+    bs.native_token_major = false;
     if (BMODE == MLK_B_NATIVE) {
         bs.native_tile_stride = (size_t)mb_total * 512;
         bs.row[0] = p.B + (size_t)p.cb0 * 512;

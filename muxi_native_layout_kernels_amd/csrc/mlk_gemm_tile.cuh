@@ -37,22 +37,34 @@ __device__ __forceinline__ WeightFrag<FP8> load_weight_frag(const uint8_t *rg_ba
     return f;
 }
 
-template <bool FP8>
-__device__ __forceinline__ u32x4 weight_operand(const WeightFrag<FP8> &f, float scale) {
+// R weight fragments of one k tile -> MFMA operands.  For fp8, `scale[r]` is the (wave-uniform)
+// block scale of stream r; one scalar test picks the short power-of-two road for the whole tile.
+template <bool FP8, int R>
+__device__ __forceinline__ void weight_operands(u32x4 (&a)[R], const WeightFrag<FP8> (&f)[R], const float (&scale)[R]) {
     if constexpr (FP8) {
-        u32x4 o;
-        uint32_t a, b, c, d;
-        if (scale_is_pow2(scale)) {
-            fp8x4_to_bf16x4_pow2(f.v[0], scale, a, b);
-            fp8x4_to_bf16x4_pow2(f.v[1], scale, c, d);
+        bool pow2 = true;
+#pragma unroll
+        for (int r = 0; r < R; ++r) pow2 = pow2 && scale_is_pow2(scale[r]);
+        if (pow2) {
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                uint32_t x0, x1, x2, x3;
+                fp8x4_to_bf16x4_pow2(f[r].v[0], scale[r], x0, x1);
+                fp8x4_to_bf16x4_pow2(f[r].v[1], scale[r], x2, x3);
+                a[r] = u32x4{x0, x1, x2, x3};
+            }
         } else {
-            fp8x4_to_bf16x4(f.v[0], scale, a, b);
-            fp8x4_to_bf16x4(f.v[1], scale, c, d);
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                uint32_t x0, x1, x2, x3;
+                fp8x4_to_bf16x4(f[r].v[0], scale[r], x0, x1);
+                fp8x4_to_bf16x4(f[r].v[1], scale[r], x2, x3);
+                a[r] = u32x4{x0, x1, x2, x3};
+            }
         }
-        o[0] = a; o[1] = b; o[2] = c; o[3] = d;
-        return o;
     } else {
-        return f.v;
+#pragma unroll
+        for (int r = 0; r < R; ++r) a[r] = f[r].v;
     }
 }
 

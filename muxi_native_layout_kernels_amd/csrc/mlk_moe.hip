@@ -11,8 +11,9 @@
 //               walk: (expert, first block, number of blocks <= CB).
 //   gate/up     grid (row tile, task): streams the gate rows and the matching
 //               up rows of W1[expert] once, gathers the task's tokens as MFMA
-//               activation fragments, and stores T(silu(gate) * up) in
-//               layout-B so the second GeMM reads it with coalesced loads
+//               activation fragments, and stores T(silu(gate) * up) as MFMA
+//               activation fragments (token-major inside a block) so the second
+//               GeMM reads only the real tokens, 64 contiguous bytes each
 //   down        grid (row tile): walks ALL tasks, streams W2[expert] rows, and
 //               adds routing weight * product into an fp32 [tokens x rows] tile
 //               in LDS; one rounding to T at the end.  This is the weighted
@@ -282,6 +283,14 @@ __global__ void __launch_bounds__(1024) moe_align_kernel(const int32_t *__restri
 }
 
 // ------------------------------------------------------------ grouped GeMMs
+// The SiLU intermediate between the two GeMMs is private to this file.  It is kept as MFMA
+// activation fragments with the token index outermost inside a block:
+// [k tile = n/32][token block][token 16][k octet 4][8 elements], so the four octets of one token
+// are 64 contiguous bytes and a block that holds only c real tokens is read as c*64 bytes.
+__device__ __forceinline__ size_t hbuf_offset(int n, int block, int token, int SB) {
+    return ((((size_t)(n >> 5) * SB + block) * 16 + token) * 4 + ((n & 31) >> 3)) * 8 + (n & 7);
+}
+
 struct MoeArgs {
     const uint8_t *W1;        // [E][2I][H] layout-A slabs
     const uint8_t *W2;        // [E][H][I]
@@ -394,11 +403,13 @@ __global__ void __launch_bounds__(max_threads_for_tiles(2 * P * CB)) moe_gate_up
     // Padding slots and blocks beyond the task read token 0: their columns of the product are
     // written to padding rows of the intermediate (or not at all) and never reach the output.
     const uint16_t *bptr[CB];
+    bool real[CB];     // lanes of padding slots issue no activation loads at all
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
         int id = p.n_pairs;
         if (cb < tk.nblocks) id = sorted[(tk.block0 + cb) * 16 + r16];
-        bptr[cb] = p.X + (size_t)(id < p.n_pairs ? id / p.K : 0) * p.H + q * 8;
+        real[cb] = id < p.n_pairs;
+        bptr[cb] = p.X + (size_t)(real[cb] ? id / p.K : 0) * p.H + q * 8;
     }
 
     f32x4 acc[R][CB];
@@ -410,20 +421,24 @@ __global__ void __launch_bounds__(max_threads_for_tiles(2 * P * CB)) moe_gate_up
     const int nt = (wave < tiles_total) ? (tiles_total - wave + p.WK - 1) / p.WK : 0;
     WeightFrag<FP8> wf[U][R];
     u32x4 bf[U][CB];
-    float sc[U][R];
+    float sc[U][2];     // block scales of the gate rows and of the up rows
     auto issue = [&](int slot, int kt) {
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-            wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
-            if (FP8) sc[slot][r] = scale_at(srows[r & 1], kt >> 2);
+        for (int r = 0; r < R; ++r) wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
+        if (FP8) {
+            sc[slot][0] = scale_at(srows[0], kt >> 2);
+            sc[slot][1] = scale_at(srows[1], kt >> 2);
         }
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * 32);
+        for (int cb = 0; cb < CB; ++cb)
+            if (real[cb]) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * 32);
     };
     auto consume = [&](int slot) {
         u32x4 a[R], b[CB];
+        float sv[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) a[r] = weight_operand<FP8>(wf[slot][r], FP8 ? sc[slot][r] : 1.f);
+        for (int r = 0; r < R; ++r) sv[r] = FP8 ? sc[slot][r & 1] : 1.f;
+        weight_operands<FP8, R>(a, wf[slot], sv);
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) b[cb] = bf[slot][cb];
 #pragma unroll
@@ -483,8 +498,7 @@ __global__ void __launch_bounds__(max_threads_for_tiles(2 * P * CB)) moe_gate_up
 #pragma unroll
         for (int i = 0; i < 4; ++i) h[i] = g[i] / (1.f + __expf(-g[i])) * u[i];
         const int n = (g0 + pr) * 16 + 4 * q;           // intermediate index = k of the down projection
-        const size_t off =
-            ((((size_t)(n >> 5) * p.SB + (tk.block0 + cb)) * 4 + ((n & 31) >> 3)) * 16 + r16) * 8 + (n & 7);
+        const size_t off = hbuf_offset(n, tk.block0 + cb, r16, p.SB);
         store4<T>(p.Hbuf + off, h[0], h[1], h[2], h[3]);
     }
 }
@@ -544,9 +558,12 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
             srow = load_scale_row(
                 p.S2 ? p.S2 + ((size_t)tk.expert * (p.H >> 7) + (rg0 >> 3)) * scale_cols : nullptr, scale_cols, lane);
         const uint16_t *bptr[CB];
+        bool real[CB];     // lanes of padding slots issue no activation loads at all
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb)
-            bptr[cb] = p.Hbuf + ((size_t)(tk.block0 + (cb < tk.nblocks ? cb : 0)) * 64 + lane) * 8;
+        for (int cb = 0; cb < CB; ++cb) {
+            real[cb] = busy && cb < tk.nblocks && sorted[(tk.block0 + cb) * 16 + r16] < p.n_pairs;
+            bptr[cb] = p.Hbuf + ((size_t)(tk.block0 + (cb < tk.nblocks ? cb : 0)) * 64 + r16 * 4 + q) * 8;
+        }
         const size_t bstep = (size_t)p.SB * 512;
 
         f32x4 acc[R][CB];
@@ -556,20 +573,21 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
             for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
         WeightFrag<FP8> wf[U][R];
         u32x4 bf[U][CB];
-        float sc[U][R];
+        float sc[U];
         auto issue = [&](int slot, int kt) {
 #pragma unroll
-            for (int r = 0; r < R; ++r) {
-                wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
-                if (FP8) sc[slot][r] = scale_at(srow, kt >> 2);
-            }
+            for (int r = 0; r < R; ++r) wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
+            if (FP8) sc[slot] = scale_at(srow, kt >> 2);
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * bstep);
+            for (int cb = 0; cb < CB; ++cb)
+                if (real[cb]) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * bstep);
         };
         auto consume = [&](int slot) {
             u32x4 a[R], b[CB];
+            float sv[R];
 #pragma unroll
-            for (int r = 0; r < R; ++r) a[r] = weight_operand<FP8>(wf[slot][r], FP8 ? sc[slot][r] : 1.f);
+            for (int r = 0; r < R; ++r) sv[r] = FP8 ? sc[slot] : 1.f;
+            weight_operands<FP8, R>(a, wf[slot], sv);
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) b[cb] = bf[slot][cb];
 #pragma unroll
@@ -673,6 +691,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_tile_kernel(MoeArgs p) {
     }
     TileBSource<CB> bs;
     bs.native_tile_stride = 0;
+    bs.native_token_major = false;
 #pragma unroll
     for (int i = 0; i < tile_granules_per_thread<CB>(); ++i) {
         int block, token, colg;
@@ -697,8 +716,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_tile_kernel(MoeArgs p) {
             for (int i = 0; i < 4; ++i)
                 h[i] = acc[2 * pr][cb][i] / (1.f + __expf(-acc[2 * pr][cb][i])) * acc[2 * pr + 1][cb][i];
             const int n = (g0 + pr) * 16 + 4 * q;
-            const size_t off =
-                ((((size_t)(n >> 5) * p.SB + (tk.block0 + cb)) * 4 + ((n & 31) >> 3)) * 16 + r16) * 8 + (n & 7);
+            const size_t off = hbuf_offset(n, tk.block0 + cb, r16, p.SB);
             store4<T>(p.Hbuf + off, h[0], h[1], h[2], h[3]);
         }
 }
@@ -732,6 +750,7 @@ __global__ void __launch_bounds__(256) moe_down_tile_kernel(MoeArgs p, float *__
     TileBSource<CB> bs;
     bs.native_tile_stride = (size_t)p.SB * 512;
     bs.row[0] = p.Hbuf + (size_t)tk.block0 * 512;          // CB consecutive blocks; those past the task are never used
+    bs.native_token_major = true;
     f32x4 acc[R][CB];
 #pragma unroll
     for (int r = 0; r < R; ++r)

@@ -56,6 +56,7 @@ template <int CB>
 struct TileBSource {
     const uint16_t *row[tile_granules_per_thread<CB>()];  // native: only row[0] = base of the first block
     size_t native_tile_stride;  // native: elements between k tiles (MB_total * 512); 0 selects row sources
+    bool native_token_major;    // native: granule order inside a block is [token][octet] instead of [octet][token]
 };
 
 template <class T, bool FP8, int CB, int R>
@@ -103,8 +104,8 @@ struct TileLoop {
                     w = g / (64 * CB);
                     const int rem = g - w * (64 * CB);
                     cb = rem >> 6;
-                    qq = (rem >> 4) & 3;
-                    rr = rem & 15;
+                    qq = bs.native_token_major ? (rem & 3) : ((rem >> 4) & 3);
+                    rr = bs.native_token_major ? ((rem >> 2) & 15) : (rem & 15);
                 } else {
                     int colg;
                     tile_row_of<CB>(i, tid, cb, rr, colg);
@@ -124,7 +125,7 @@ struct TileLoop {
 #pragma unroll
                 for (int r = 0; r < R; ++r) {
                     wf[slot][w][r] = load_weight_frag<FP8>(abase[r], tile0 + w, lane);
-                    if (FP8) sc[slot][w][r] = scale_at(srow[r], (tile0 + w) >> 2);
+                    sc[slot][w][r] = FP8 ? scale_at(srow[r], (tile0 + w) >> 2) : 1.f;
                 }
         };
         auto step = [&](int slot, bool do_stage, bool do_issue) {
@@ -134,8 +135,7 @@ struct TileLoop {
                 u32x4 b[CB], a[R];
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) b[cb] = win[slot * WG + (w * CB + cb) * 68 + q * 17 + r16];
-#pragma unroll
-                for (int r = 0; r < R; ++r) a[r] = weight_operand<FP8>(wf[slot][w][r], FP8 ? sc[slot][w][r] : 1.f);
+                weight_operands<FP8, R>(a, wf[slot][w], sc[slot][w]);
 #pragma unroll
                 for (int r = 0; r < R; ++r)
 #pragma unroll
