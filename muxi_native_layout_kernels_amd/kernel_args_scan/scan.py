@@ -33,7 +33,7 @@ DEFAULT_SHAPES = {
     "gemv_bf16": [(4096, 4096), (28672, 8192), (8192, 8192), (28672, 4096), (4096, 14336)],
     "gemv_soft_fp8": [(28672, 8192), (4096, 4096), (8192, 8192)],
     "layoutA_gemm": [(11008, 4096), (4096, 4096), (4096, 11008)],
-    "layoutA_soft_fp8_gemm": [(28672, 8192)],
+    "layoutA_soft_fp8_gemm": [(28672, 8192), (4096, 4096)],
     "continuous_gemm": [(8192, 8192), (11008, 4096)],
     "layout_gemm": [(8192, 8192), (11008, 4096)],
 }
@@ -134,19 +134,23 @@ def scan_gemm(table, shapes, tokens, iters):
             want = b.float() @ w0.t()
             b_in = ops.layoutB(b) if mode in ("continuous", "native") else b
             best = None
-            for p1 in (1, 2, 4):
+            grid = [(1, r, w, sk) for r in (1, 2, 4) for w in (1, 2, 4, 8, 16) for sk in ((1, 2, 4) if n <= 8192 else (1,))]
+            # kernel 2 (row-shared tiles): 4 waves x p1 row groups per workgroup, K split only across workgroups
+            grid += [(2, r, 1, sk) for r in (1, 2, 4) for sk in (1, 2, 4, 8)
+                     if (n // 16) % (4 * r) == 0 and (k // 32) % (4 * sk) == 0 and m > 16]
+            for kid, p1, p2, p3 in grid:
                 if (n // 16) % p1:
                     continue
-                for p2, p3 in [(w, sk) for w in (1, 2, 4, 8, 16) for sk in ((1, 2, 4) if n <= 8192 else (1,))]:
+                if True:
                     def call(a):
                         if mode == "rowmajor":
-                            return lambda: ops.gemm_layoutA_wapper(a, b_in, n, m, k, 1, 0, p1, p2, p3, 1, None)
+                            return lambda: ops.gemm_layoutA_wapper(a, b_in, n, m, k, 1, 0, p1, p2, p3, kid, None)
                         if mode == "fp8":
-                            return lambda: ops.gemm_layoutA_soft_fp8_wapper(a, scale, b_in, n, m, k, 1, 0, p1, p2, p3, 1,
+                            return lambda: ops.gemm_layoutA_soft_fp8_wapper(a, scale, b_in, n, m, k, 1, 0, p1, p2, p3, kid,
                                                                             None)
                         if mode == "continuous":
-                            return lambda: ops.gemm_layoutAB_ContinuousC_wapper(a, b_in, n, m, k, 1, 0, p1, p2, p3, 1, None)
-                        return lambda: ops.gemm_layoutABC_wapper(a, b_in, n, m, k, 1, 0, p1, p2, p3, 1, None)
+                            return lambda: ops.gemm_layoutAB_ContinuousC_wapper(a, b_in, n, m, k, 1, 0, p1, p2, p3, kid, None)
+                        return lambda: ops.gemm_layoutABC_wapper(a, b_in, n, m, k, 1, 0, p1, p2, p3, kid, None)
                     got = call(packed[0])()
                     if mode == "native":
                         got = ops.reLayoutC(got)
@@ -154,7 +158,7 @@ def scan_gemm(table, shapes, tokens, iters):
                         continue
                     us = _time_graph([call(a) for a in packed], iters)
                     if best is None or us < best[0]:
-                        best = (us, 1, p1, p2, p3)
+                        best = (us, kid, p1, p2, p3)
             print("%s %dx%d M=%d -> %s" % (table, n, k, m, best), file=sys.stderr)
             rows.append("%d,%d,%d,%d,%d,%d,%d" % (n, m, k, best[1], best[2], best[3], best[4]))
         del plain, packed

@@ -70,3 +70,17 @@ def test_relayout_errors(mlk):
         mlk.layoutB(torch.zeros(16, 32, dtype=torch.bfloat16))
     empty = mlk.layoutB(torch.zeros(0, 32, dtype=torch.bfloat16, device="cuda"))
     assert empty.shape == (1, 0, 4, 16, 8)
+
+
+def test_stream_read_probe(mlk):
+    """The measurement aid reads a buffer and writes nothing; it must accept any divisor grid."""
+    from muxi_native_layout_kernels_amd import _lib
+    lib = _lib.load()
+    buf = torch.randint(0, 255, (8 << 20,), dtype=torch.uint8, device="cuda")
+    keep = buf.clone()
+    st = torch.cuda.current_stream().cuda_stream
+    for block, wgs in ((256, 1024), (1024, 64), (64, 8192)):
+        assert lib.mlk_stream_read(buf.data_ptr(), buf.numel(), block, wgs, None, st) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(buf, keep)
+    assert lib.mlk_stream_read(buf.data_ptr(), buf.numel(), 256, 1000, None, st) == -1   # 8192 tiles % 1000 != 0
