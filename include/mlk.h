@@ -47,11 +47,18 @@ extern "C" {
 int mlk_version(void);
 const char *mlk_last_error(void);
 /* Experiment switches for the tuning scripts (process-wide, not thread-safe):
- * id 0 = rotate the k-tile visiting order of the narrow GeMM per row tile (default 1).
+ *   id 0  rotate the k-tile visiting order of the narrow GeMM per row tile (default 1)
+ *   id 1  stage row-major activations of the wave GeMM kernel through LDS when more than
+ *         32 tokens share a weight pass (default 1)
+ *   id 2, 3  single-token MoE, gate/up kernel: row groups per workgroup and waves splitting K
+ *         (defaults 1 and 8; 2 * id2 * id3 <= 16)
+ *   id 4  single-token MoE, down kernel: waves per workgroup (default 16)
+ *   id 5  single-token MoE: 16-byte loads in flight per wave, 2, 3, 4, 6 or 8 (default 4)
  * No counterpart in the reference. */
 void mlk_set_tunable(int id, int value);
-/* Experiment switch: use (1, default) or avoid (0) the row-shared kernels of the fused MoE for
- * more than 16 tokens.  No counterpart in the reference. */
+/* Experiment switches of the fused MoE: bit 0 set (default) = use the row-shared kernels for more
+ * than 16 tokens, bit 1 set = do NOT use the single-token GeMV kernels.  Default 1.
+ * No counterpart in the reference. */
 void mlk_moe_set_tile_path(int on);
 
 /* ------------------------------------------------------------------ relayout
@@ -98,8 +105,9 @@ int mlk_stream_read(const void *src, int64_t nbytes, int block_dim_x, int workgr
  * Launch parameters (what the reference's csv rows select):
  *   block_dim_x  threads per workgroup, 64..1024, multiple of 64
  *   kernel_id    1 = streaming kernel (the only one)
- *   p1           row groups (of 16 rows) per workgroup, >= 1, divides N/16... see DESIGN
- *   p2           loads kept in flight per wave, 1..8
+ *   p1           row groups (of 16 rows) per workgroup: >= 1 and divides both N/16 and
+ *                block_dim_x/64; the block_dim_x/64/p1 waves of a row group split K
+ *   p2           16-byte loads kept in flight per wave: 1, 2, 4, 6 or 8
  */
 int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k, int a_kind, int x_kind,
                       float alpha, const void *bias, const float *scale, int block_dim_x, int kernel_id, int p1,
@@ -120,9 +128,15 @@ int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k
  *
  * With a native B or C, M must be a multiple of 16.  N % 16 == 0, K % 32 == 0
  * (K % 64 == 0 for fp8 weights; N % 32 == 0 for a native C).
- * Launch parameters: kernel_id 1; p1 = row groups per wave (1, 2 or 4);
- * p2 = waves per workgroup that split K (1, 2, 4, 8 or 16); p3 = K splits across
- * workgroups (>= 1; > 1 needs `workspace`).
+ * Launch parameters:
+ *   kernel_id 1  wave kernel: every wave owns p1 row groups and gathers its own activations;
+ *                p2 = waves per workgroup that split K (1, 2, 4, 8 or 16)
+ *   kernel_id 2  row-shared kernel: four waves walk the same k tiles and share the activations
+ *                of each k window through LDS (p2 is ignored); falls back to kernel 1 for a
+ *                shape it does not tile (N/16 not a multiple of 4 p1, or K/32 not a multiple
+ *                of 4 p3)
+ *   p1 = row groups per wave (1, 2 or 4); p3 = K splits across workgroups (>= 1; > 1 needs
+ *   `workspace`).
  * workspace: device scratch of at least mlk_gemm_workspace_bytes() bytes, only
  * read and written inside the call (contents need not be preserved, but the
  * first `mlk_gemm_counter_bytes()` bytes must be zero before the first call and

@@ -27,7 +27,7 @@ constexpr size_t kCounterBytes = 64 * 1024;
 
 // Experiment switches (mlk_set_tunable): [0] rotate the k-tile order per row tile,
 // [1] stage row-major activations through LDS.
-static int g_tunable[8] = {1, 1, 0, 0, 0, 0, 0, 0};
+int g_tunable[8] = {1, 1, 1, 8, 16, 4, 0, 0};
 
 struct GemmArgs {
     const uint8_t *A;

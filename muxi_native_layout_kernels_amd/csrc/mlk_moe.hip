@@ -30,6 +30,7 @@ namespace mlk {
 constexpr int kMaxExperts = 256;
 constexpr int kMaxTopK = 32;
 constexpr int kMoeChunk = 256;     // tokens per expert-compute pass
+static int g_moe_gemv1 = 1;        // experiment switch: GeMV-style kernels for a single token
 static int g_moe_tile = 1;         // experiment switch: row-shared kernels for tasks of more than one token block
 static inline bool moe_tile_path() { return g_moe_tile != 0; }
 // Token blocks per task: as many as the largest possible expert load needs, at most 8 with the
@@ -658,6 +659,207 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
     }
 }
 
+// ------------------------------------------------------- single-token variants (one token)
+// With one token every routed pair is a GeMV.  These two kernels stream the expert rows like the
+// GeMV kernel (16-byte loads, register ring, v_dot2, no MFMA) with the activation vector in LDS,
+// so nothing but weights crosses the memory system.
+
+// One tile of weights (1 KiB: 16 rows x 32 k, or 16 rows x 64 k for fp8) times the matching
+// activations in LDS.  acc[0] is the lane's row (row lane&15; for fp8 row 2*(lane&7)), acc[1] the
+// second fp8 row.
+template <class T, bool FP8>
+__device__ __forceinline__ void gemv1_tile(const u32x4 &w, float s, const u32x4 *xs, int granule, float (&acc)[2]) {
+    const u32x4 xv = xs[granule];
+    if (FP8) {
+        uint32_t w0[4], w1[4];
+        if (scale_is_pow2(s)) {
+            fp8x4_to_bf16x4_pow2(w[0], s, w0[0], w0[1]);
+            fp8x4_to_bf16x4_pow2(w[1], s, w0[2], w0[3]);
+            fp8x4_to_bf16x4_pow2(w[2], s, w1[0], w1[1]);
+            fp8x4_to_bf16x4_pow2(w[3], s, w1[2], w1[3]);
+        } else {
+            fp8x4_to_bf16x4(w[0], s, w0[0], w0[1]);
+            fp8x4_to_bf16x4(w[1], s, w0[2], w0[3]);
+            fp8x4_to_bf16x4(w[2], s, w1[0], w1[1]);
+            fp8x4_to_bf16x4(w[3], s, w1[2], w1[3]);
+        }
+#pragma unroll
+        for (int d = 0; d < 4; ++d) {
+            acc[0] = T::dot2(w0[d], xv[d], acc[0]);
+            acc[1] = T::dot2(w1[d], xv[d], acc[1]);
+        }
+    } else {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) acc[0] = T::dot2(w[d], xv[d], acc[0]);
+    }
+}
+
+// The tiles ks, ks + WK, ... of one row group against an activation vector in LDS.  The first
+// weight loads are put in flight, then `stage` runs (the caller copies the activations to LDS and
+// synchronises the workgroup there), then the rest streams; the 16 row sums end in red16[0..15].
+template <class T, bool FP8, int U, class Stage>
+__device__ __forceinline__ void gemv1_stream(const uint8_t *rowgroup, int tiles, int ks, int WK, const u32x4 *xs,
+                                             const ScaleRow &srow, float *red16, Stage stage) {
+    constexpr int TKG = FP8 ? 8 : 4;                 // activation granules (8 elements) per tile
+    const int lane = threadIdx.x & 63;
+    const int oct = FP8 ? (lane >> 3) : (lane >> 4);
+    const u32x4 *ap = reinterpret_cast<const u32x4 *>(rowgroup) + (size_t)ks * 64 + lane;
+    const int stride = WK * 64;
+    const int nt = ks < tiles ? (tiles - ks + WK - 1) / WK : 0;
+    float acc[2] = {0.f, 0.f};
+    u32x4 buf[U];
+    float sc[U];
+    auto issue = [&](int u, int j) {
+        buf[u] = ld_stream_u32x4(ap + (size_t)j * stride);
+        sc[u] = FP8 ? scale_at(srow, (ks + j * WK) >> 1) : 1.f;
+    };
+    auto consume = [&](int u, int j) { gemv1_tile<T, FP8>(buf[u], sc[u], xs, (ks + j * WK) * TKG + oct, acc); };
+    const bool full = nt >= U;
+    if (full) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) issue(u, u);
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < nt) issue(u, u);
+    }
+    stage();
+    if (full) {
+        int i = 0;
+        for (; i + 2 * U <= nt; i += U) {
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                consume(u, i + u);
+                issue(u, i + U + u);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        }
+        const int rem = nt - i - U;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            consume(u, i + u);
+            if (u < rem) issue(u, i + U + u);
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < rem) consume(u, i + U + u);
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (u < nt) consume(u, u);
+    }
+#pragma unroll
+    for (int a = 0; a < (FP8 ? 2 : 1); ++a) {
+        float v = acc[a];
+        if (FP8) v += lane_xor(v, 8);
+        v += lane_xor(v, 16);
+        v += lane_xor(v, 32);
+        acc[a] = v;
+    }
+    if (FP8) {
+        if (lane < 8) {
+            red16[2 * lane] = acc[0];
+            red16[2 * lane + 1] = acc[1];
+        }
+    } else if (lane < 16) {
+        red16[lane] = acc[0];
+    }
+}
+
+struct Moe1Args {
+    const uint8_t *W1, *W2;
+    const float *S1, *S2;
+    const uint16_t *X;        // [H]
+    uint16_t *Y;              // [H]
+    uint16_t *Hd;             // [K][I] intermediate
+    const uint16_t *wts;      // [K]
+    const int32_t *topk_ids;  // [K]
+    const int32_t *experts_map;
+    int K, H, I, E;
+    int G, WK;                // gate/up: row groups per workgroup and waves splitting K (2*G*WK waves)
+    int DW;                   // down: waves per workgroup
+};
+
+// gate/up for one token: grid (I/(16 G), K); waves = (gate, up) x G row groups x WK slices of K
+template <class T, bool FP8, int U>
+__global__ void __launch_bounds__(1024) moe_gate_up_gemv1_kernel(Moe1Args p) {
+    extern __shared__ u32x4 xs[];          // the token's hidden vector
+    __shared__ float red[16][16];
+    int e = p.topk_ids[blockIdx.y];
+    if (p.experts_map) e = p.experts_map[e];
+    if (e < 0 || e >= p.E) return;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int stream = wave / (p.G * p.WK);
+    const int gl = (wave / p.WK) % p.G, ks = wave % p.WK;
+    constexpr int WB = FP8 ? 1 : 2;
+    constexpr int TK = FP8 ? 64 : 32;
+    const int col = blockIdx.x * p.G + gl;                 // 16-column group of the intermediate
+    const int rg = stream * (p.I >> 4) + col;
+    const uint8_t *rowgroup = p.W1 + (size_t)e * 2 * p.I * p.H * WB + (size_t)rg * p.H * 16 * WB;
+    ScaleRow srow;
+    if (FP8)
+        srow = load_scale_row(p.S1 ? p.S1 + ((size_t)e * (2 * p.I >> 7) + (rg >> 3)) * (p.H >> 7) : nullptr, p.H >> 7, lane);
+    gemv1_stream<T, FP8, U>(rowgroup, p.H / TK, ks, p.WK, xs, srow, red[wave], [&]() {
+        for (int i = threadIdx.x; i < (p.H >> 3); i += blockDim.x) xs[i] = reinterpret_cast<const u32x4 *>(p.X)[i];
+        __syncthreads();
+    });
+    __syncthreads();
+    if (threadIdx.x < 16 * p.G) {
+        const int g_local = threadIdx.x >> 4, r = threadIdx.x & 15;
+        float g = 0.f, u = 0.f;
+        for (int w = 0; w < p.WK; ++w) {
+            g += red[g_local * p.WK + w][r];
+            u += red[(p.G + g_local) * p.WK + w][r];
+        }
+        const float h = g / (1.f + __expf(-g)) * u;
+        p.Hd[(size_t)blockIdx.y * p.I + (blockIdx.x * p.G + g_local) * 16 + r] = (uint16_t)T::from_f32(h);
+    }
+}
+
+// down for one token: grid (H/16); the DW waves are dealt to the K pairs, DW/K slices of K each
+template <class T, bool FP8, int U>
+__global__ void __launch_bounds__(1024) moe_down_gemv1_kernel(Moe1Args p) {
+    extern __shared__ u32x4 hs[];          // [K][I/8] intermediates of all pairs
+    __shared__ float red[16][16];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    constexpr int WB = FP8 ? 1 : 2;
+    constexpr int TK = FP8 ? 64 : 32;
+    const int wpt = p.DW / p.K;            // host: K <= DW
+    const int pair = wave / wpt, ks = wave - pair * wpt;
+    const int gran = p.I >> 3;
+    int e = -1;
+    if (pair < p.K) {
+        e = p.topk_ids[pair];
+        if (p.experts_map) e = p.experts_map[e];
+        if (e >= p.E) e = -1;
+    }
+    // a wave without work (absent expert) streams zero tiles and leaves zero sums
+    const int ee = e >= 0 ? e : 0;
+    const uint8_t *rowgroup = p.W2 + (size_t)ee * p.H * p.I * WB + (size_t)blockIdx.x * p.I * 16 * WB;
+    ScaleRow srow;
+    if (FP8)
+        srow = load_scale_row(p.S2 ? p.S2 + ((size_t)ee * (p.H >> 7) + (blockIdx.x >> 3)) * (p.I >> 7) : nullptr,
+                              p.I >> 7, lane);
+    gemv1_stream<T, FP8, U>(rowgroup, e >= 0 ? p.I / TK : 0, ks, wpt, hs + (size_t)(pair < p.K ? pair : 0) * gran, srow,
+                            red[wave], [&]() {
+                                for (int i = threadIdx.x; i < p.K * gran; i += blockDim.x)
+                                    hs[i] = reinterpret_cast<const u32x4 *>(p.Hd)[i];
+                                __syncthreads();
+                            });
+    __syncthreads();
+    if (threadIdx.x < 16) {
+        float y = 0.f;
+        for (int k = 0; k < p.K; ++k) {          // pick order; pairs of absent experts left zeros
+            float s = 0.f;
+            for (int w = 0; w < wpt; ++w) s += red[k * wpt + w][threadIdx.x];
+            y += T::to_f32(p.wts[k]) * s;
+        }
+        p.Y[blockIdx.x * 16 + threadIdx.x] = (uint16_t)T::from_f32(y);
+    }
+}
+
 // ------------------------------------------------ row-shared variants (more than 16 tokens)
 // For tasks of two to four token blocks the four waves of a workgroup share the activation
 // windows through LDS (mlk_tile.cuh) instead of gathering them per wave.
@@ -909,7 +1111,10 @@ static int launch_moe_cb(const MoeArgs &a, int cb, int max_tasks, bool inline_al
 
 using namespace mlk;
 
-extern "C" void mlk_moe_set_tile_path(int on) { g_moe_tile = on; }
+extern "C" void mlk_moe_set_tile_path(int on) {
+    g_moe_tile = on & 1;
+    g_moe_gemv1 = (on >> 1) & 1 ? 0 : 1;       // bit 1 switches the single-token kernels off
+}
 
 extern "C" int mlk_fused_routing_gate(const void *logits, int x_kind, int score_fun, int n_tokens, int n_experts,
                                       int n_groups, int topk_groups, int topk, const void *bias, int renormalize,
@@ -989,6 +1194,56 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
         if (max_blocks < kDecodePairs) max_blocks = kDecodePairs;
         const int active = n_experts < n_pairs ? n_experts : n_pairs;
         const int max_tasks = active + n_pairs / (16 * cb);
+        // one token: every routed pair is a GeMV with the activations in LDS
+        if (g_moe_gemv1 && tc == 1 && topk <= 16 && (size_t)topk * inter * 2 <= 56 * 1024 &&
+            (size_t)hidden * 2 <= 56 * 1024 && (!fp8 || (hidden % 64 == 0 && inter % 64 == 0))) {
+            Moe1Args m;
+            m.W1 = (const uint8_t *)w1;
+            m.W2 = (const uint8_t *)w2;
+            m.S1 = w1_scale;
+            m.S2 = w2_scale;
+            m.X = (const uint16_t *)x + (size_t)t0 * hidden;
+            m.Y = (uint16_t *)y + (size_t)t0 * hidden;
+            m.Hd = ws.hbuf;
+            m.wts = (const uint16_t *)topk_weights + (size_t)t0 * topk;
+            m.topk_ids = topk_ids + (size_t)t0 * topk;
+            m.experts_map = experts_map;
+            m.K = topk;
+            m.H = hidden;
+            m.I = inter;
+            m.E = n_experts;
+            // tunables 2..5: G, WK of the gate/up kernel, waves of the down kernel, loads in flight
+            int G = g_tunable[2], WK = g_tunable[3], DW = g_tunable[4];
+            if (G < 1 || WK < 1 || 2 * G * WK > 16 || (inter / 16) % G) G = 1, WK = 8;
+            if (DW < topk || DW > 16) DW = 16;
+            DW -= DW % topk;
+            m.G = G;
+            m.WK = WK;
+            m.DW = DW;
+            const dim3 g1(inter / (16 * G), topk), g2(hidden / 16);
+            const int b1 = 2 * G * WK * 64, b2 = DW * 64;
+            const size_t l1 = (size_t)hidden * 2, l2 = (size_t)topk * inter * 2;
+#define MLK_MOE1(TT, F8, UU)                                                        \
+    do {                                                                            \
+        moe_gate_up_gemv1_kernel<TT, F8, UU><<<g1, b1, l1, s>>>(m);                 \
+        moe_down_gemv1_kernel<TT, F8, UU><<<g2, b2, l2, s>>>(m);                    \
+    } while (0)
+#define MLK_MOE1_U(TT, F8)                                                          \
+    do {                                                                            \
+        if (g_tunable[5] == 2) MLK_MOE1(TT, F8, 2);                                 \
+        else if (g_tunable[5] == 3) MLK_MOE1(TT, F8, 3);                            \
+        else if (g_tunable[5] == 6) MLK_MOE1(TT, F8, 6);                            \
+        else if (g_tunable[5] == 8) MLK_MOE1(TT, F8, 8);                            \
+        else MLK_MOE1(TT, F8, 4);                                                   \
+    } while (0)
+            if (fp8) MLK_MOE1_U(BF16, true);
+            else if (x_kind == MLK_F16) MLK_MOE1_U(F16, false);
+            else MLK_MOE1_U(BF16, false);
+#undef MLK_MOE1_U
+#undef MLK_MOE1
+            MLK_LAUNCH_CHECK();
+            continue;
+        }
         // decode-sized batches align inside the GeMM kernels; larger ones run the alignment kernel
         const bool inline_align = tc <= 16 && n_pairs <= kDecodePairs;
         if (!inline_align) {

@@ -17,7 +17,6 @@ from . import _lib, arg_selector
 
 _KIND = {torch.float16: 0, torch.bfloat16: 1}
 _FP8_KIND = 2
-_BYTE_DTYPES = (torch.uint8, torch.int8, getattr(torch, "float8_e4m3fn", torch.uint8))
 
 
 def _stream():

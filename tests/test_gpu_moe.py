@@ -184,6 +184,44 @@ def test_fused_moe_expert_map(mlk):
     assert_close(y, want, RTOL, ATOL, "expert map")
 
 
+@pytest.mark.parametrize("dtype,fp8,E,K,H,I", [
+    (torch.float16, False, 8, 2, 256, 384),
+    (torch.bfloat16, False, 16, 6, 512, 256),
+    (torch.bfloat16, True, 16, 8, 384, 512),
+    (torch.bfloat16, False, 64, 16, 128, 128),
+    (torch.bfloat16, False, 32, 20, 256, 128),      # top-k above 16: the general decode kernels
+])
+def test_fused_moe_single_token(mlk, dtype, fp8, E, K, H, I):
+    """One token runs GeMV-style kernels; switching them off must give the grouped kernels' result
+    to the same tolerance."""
+    from muxi_native_layout_kernels_amd import _lib
+    y1 = _moe_case(mlk, 1, E, K, H, I, dtype, 900 + K, fp8=fp8)
+    _lib.load().mlk_moe_set_tile_path(3)
+    try:
+        y2 = _moe_case(mlk, 1, E, K, H, I, dtype, 900 + K, fp8=fp8)
+    finally:
+        _lib.load().mlk_moe_set_tile_path(1)
+    assert_close(y1, y2.double().cpu().numpy(), RTOL, ATOL, "single-token kernels vs grouped kernels")
+
+
+def test_fused_moe_single_token_expert_map(mlk):
+    """A routed expert that is not held locally contributes nothing."""
+    from muxi_native_layout_kernels_amd.moe_planC import fused_moe
+    E, K, H, I = 8, 4, 256, 256
+    dtype = torch.bfloat16
+    emap = np.array([0, -1, 1, -1, 2, -1, 3, -1], dtype=np.int32)
+    w1 = randn((4, 2 * I, H), dtype, 0.02, 3)
+    w2 = randn((4, H, I), dtype, 0.02, 4)
+    w1p, w2p = _pack_experts(w1).cuda(), _pack_experts(w2).cuda()
+    for seed in range(4):
+        x = randn((1, H), dtype, 1.0, 10 + seed)
+        logits = randn((1, E), dtype, 1.0, 20 + seed)
+        y = fused_moe(x.cuda(), w1p, w2p, logits.cuda(), K, True, experts_map=torch.as_tensor(emap).cuda())
+        ids, wts = orouter.route(logits, 0, 1, 1, K)
+        want = omoe.moe_expected(x, w1, w2, ids, orouter.renormalize(wts), round_h_to=dtype, expert_map=emap)
+        assert_close(y, want, RTOL, ATOL, "single token, expert map")
+
+
 def test_fused_moe_matches_torch_path_on_gpu(mlk):
     """The reference's own test recipe: compare with the pure-torch MoE run on the GPU in the same dtype,
     atol 0.1 / rtol 0.05 (benchmark_and_test/test_muxi_moe.py:111)."""
