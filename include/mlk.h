@@ -54,6 +54,8 @@ const char *mlk_last_error(void);
  *         (defaults 1 and 8; 2 * id2 * id3 <= 16)
  *   id 4  single-token MoE, down kernel: waves per workgroup (default 16)
  *   id 5  single-token MoE: 16-byte loads in flight per wave, 2, 3, 4, 6 or 8 (default 4)
+ *   id 7  decode MoE (2..16 tokens), down kernel: row groups per wave = K slices across
+ *         workgroups, 1, 2 or 4 (default 0 = 4 for soft-FP8 weights, 1 otherwise)
  * No counterpart in the reference. */
 void mlk_set_tunable(int id, int value);
 /* Experiment switches of the fused MoE: bit 0 set (default) = use the row-shared kernels for more

@@ -307,6 +307,9 @@ struct MoeArgs {
     const int32_t *topk_ids;  // [T*K], read by the decode variants that align in-kernel
     const int32_t *experts_map;
     int T, K, H, I, SB, n_pairs, WK, E;
+    float *part;              // down projection with K slices: fp32 partial output tiles [slice][workgroup][T][16R]
+    int32_t *counters;        // arrival counters, one per down workgroup column (zeroed by the gate/up kernel)
+    int n_counters;
 };
 
 // Decode-sized batches (T*K <= 64 pairs): every workgroup rebuilds the tiny alignment itself
@@ -362,6 +365,9 @@ __global__ void __launch_bounds__(max_threads_for_tiles(2 * P * CB)) moe_gate_up
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int task = blockIdx.y;
+    // the down kernel that follows counts workgroup arrivals per output column
+    if (blockIdx.x == 0 && blockIdx.y == 0)
+        for (int i = threadIdx.x; i < p.n_counters; i += blockDim.x) p.counters[i] = 0;
     const MoeTask *tasks = p.tasks;
     const int32_t *sorted = p.sorted;
     int n_tasks;
@@ -516,6 +522,7 @@ template <class T, bool FP8, int CB, int R, int U, bool INLINE>
 __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(MoeArgs p) {
     extern __shared__ f32x4 red[];  // [WK][R*CB][64] then the fp32 output tile [T][16R]
     __shared__ DecodeTables dec;
+    __shared__ int s_last;
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const MoeTask *tasks = p.tasks;
@@ -525,7 +532,9 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
     const int rg0 = blockIdx.x * R;
     constexpr int WB = FP8 ? 1 : 2;
     constexpr int NT = R * CB;
-    const int tiles_total = p.I >> 5;
+    // blockIdx.y = K slice (the host makes the slices equal)
+    const int tiles_total = (p.I >> 5) / gridDim.y;
+    const int tbeg = blockIdx.y * tiles_total;
     const size_t slab = (size_t)p.H * p.I * WB;
     const int scale_cols = p.I >> 7;
     float *ytile = reinterpret_cast<float *>(red + (size_t)p.WK * NT * 64);
@@ -597,7 +606,7 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
                 for (int cb = 0; cb < CB; ++cb) acc[r][cb] = T::mfma(a[r], b[cb], acc[r][cb]);
         };
         int jcur = 0;
-        auto next_tile = [&]() { return ks + (jcur++) * wpt; };
+        auto next_tile = [&]() { return tbeg + ks + (jcur++) * wpt; };
         if (nt >= U) {
 #pragma unroll
             for (int u = 0; u < U; ++u) issue(u, next_tile());
@@ -653,9 +662,33 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
         base += g;
     }
 
-    for (int i = threadIdx.x; i < p.T * yrows; i += blockDim.x) {
-        int tok = i / yrows, row = i - tok * yrows;
-        p.Y[(size_t)tok * p.H + rg0 * 16 + row] = (uint16_t)T::from_f32(ytile[i]);
+    if (gridDim.y == 1) {
+        for (int i = threadIdx.x; i < p.T * yrows; i += blockDim.x) {
+            int tok = i / yrows, row = i - tok * yrows;
+            p.Y[(size_t)tok * p.H + rg0 * 16 + row] = (uint16_t)T::from_f32(ytile[i]);
+        }
+        return;
+    }
+    // K slices: publish the fp32 tile with agent-coherent stores; the last workgroup to arrive
+    // for this column folds the slices in slice order.
+    const int cells = p.T * yrows / 4;              // f32x4 cells of a tile
+    f32x4 *part = reinterpret_cast<f32x4 *>(p.part);
+    auto tile_at = [&](int sk) { return part + ((size_t)sk * gridDim.x + blockIdx.x) * cells; };
+    for (int i = threadIdx.x; i < cells; i += blockDim.x)
+        st_agent_f32x4(tile_at(blockIdx.y) + i, *reinterpret_cast<const f32x4 *>(ytile + 4 * i));
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int prev = __hip_atomic_fetch_add(&p.counters[blockIdx.x], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (prev == (int)gridDim.y - 1);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    for (int i = threadIdx.x; i < cells; i += blockDim.x) {
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        for (int sk = 0; sk < (int)gridDim.y; ++sk) v += ld_agent_f32x4(tile_at(sk) + i);
+        const int e = 4 * i, tok = e / yrows, row = e - tok * yrows;
+        store4<T>(p.Y + (size_t)tok * p.H + rg0 * 16 + row, v[0], v[1], v[2], v[3]);
     }
 }
 
@@ -1005,8 +1038,11 @@ struct MoeWorkspace {
     int32_t *sorted, *cumsum, *padded, *experts_ids;
     uint16_t *hbuf;
     float *obuf;
+    int32_t *counters;
     int sb;          // token blocks the intermediate is dimensioned for
 };
+
+constexpr int kDecodeKSlices = 4;
 
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 
@@ -1031,9 +1067,28 @@ static size_t carve(uint8_t *base, int tc, int E, int K, int hidden, int inter, 
     // seven spare blocks: the row-shared down kernel always fetches CB <= 8 consecutive blocks
     w.sb = max_blocks + 7;
     w.hbuf = (uint16_t *)take((size_t)inter * w.sb * 16 * 2);
-    w.obuf = (float *)take(tc > 16 ? (size_t)n_pairs * 8 * hidden * sizeof(float) : 0);   // 8 = kMoeMaxKSlices
+    // fp32 buffer of the K-sliced down projections: per routed pair and slice for the row-shared
+    // kernels, per token and slice (up to 4) for the decode kernel
+    w.obuf = (float *)take(tc > 16 ? (size_t)n_pairs * 8 * hidden * sizeof(float)
+                                   : (size_t)tc * kDecodeKSlices * hidden * sizeof(float));   // 8 = kMoeMaxKSlices
+    w.counters = (int32_t *)take(sizeof(int32_t) * (size_t)(hidden / 16));
     if (ws) *ws = w;
     return off;
+}
+
+template <class T, bool FP8, int CB, int R, bool INLINE>
+static int launch_moe_down(const MoeArgs &a, int skd, hipStream_t s) {
+    constexpr int U2F = (R * CB >= 4) ? 4 : (R * CB == 1 ? 10 : 6);   // fp8 tiles are half as many bytes
+    constexpr int U2 = FP8 && CB == 1 ? U2F : ((R * CB >= 4) ? 3 : (R * CB == 1 ? 8 : 4));
+    MoeArgs d = a;
+    d.WK = 16;
+    while (d.WK > 1 && (d.WK * 64 > max_threads_for_tiles(R * CB) ||
+                        (size_t)d.WK * R * CB * 1024 + (size_t)a.T * 16 * R * 4 + sizeof(DecodeTables) > 64 * 1024))
+        d.WK >>= 1;
+    size_t lds2 = (size_t)d.WK * R * CB * 1024 + (size_t)a.T * 16 * R * 4;
+    moe_down_kernel<T, FP8, CB, R, U2, INLINE><<<dim3(a.H / 16 / R, skd), d.WK * 64, lds2, s>>>(d);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
 }
 
 template <class T, bool FP8, int CB, bool INLINE>
@@ -1050,17 +1105,15 @@ static int launch_moe(const MoeArgs &a, int max_tasks, hipStream_t s) {
     moe_gate_up_kernel<T, FP8, CB, P, U1, INLINE><<<dim3(grid_x, max_tasks), g.WK * 64, lds1, s>>>(g);
     MLK_LAUNCH_CHECK();
 
-    constexpr int R = 1;
-    constexpr int U2 = (CB >= 4) ? 3 : (CB == 1 ? 8 : 4);
-    MoeArgs d = a;
-    d.WK = 16;
-    while (d.WK > 1 && (d.WK * 64 > max_threads_for_tiles(R * CB) ||
-                        (size_t)d.WK * R * CB * 1024 + (size_t)a.T * 16 * R * 4 + sizeof(DecodeTables) > 64 * 1024))
-        d.WK >>= 1;
-    size_t lds2 = (size_t)d.WK * R * CB * 1024 + (size_t)a.T * 16 * R * 4;
-    moe_down_kernel<T, FP8, CB, R, U2, INLINE><<<a.H / 16 / R, d.WK * 64, lds2, s>>>(d);
-    MLK_LAUNCH_CHECK();
-    return MLK_OK;
+    if constexpr (CB == 1) {
+        // One token block: R row groups per wave cut the re-reads of the intermediate R-fold; K is
+        // sliced R ways so that the grid still has a workgroup per 16 output rows.
+        const int r = g_tunable[7] ? g_tunable[7] : (FP8 ? 4 : 1);
+        const int tiles = a.I / 32;
+        if (r == 2 && (a.H / 16) % 2 == 0 && tiles % 2 == 0) return launch_moe_down<T, FP8, CB, 2, INLINE>(a, 2, s);
+        if (r == 4 && (a.H / 16) % 4 == 0 && tiles % 4 == 0) return launch_moe_down<T, FP8, CB, 4, INLINE>(a, 4, s);
+    }
+    return launch_moe_down<T, FP8, CB, 1, INLINE>(a, 1, s);
 }
 
 constexpr int kMoeMaxKSlices = 8;  // K slices of the row-shared down projection (sizes its fp32 buffer)
@@ -1274,6 +1327,9 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
         a.E = n_experts;
         a.topk_ids = topk_ids + (size_t)t0 * topk;
         a.experts_map = experts_map;
+        a.part = ws.obuf;
+        a.counters = ws.counters;
+        a.n_counters = hidden / 16;
         int rc;
         if (fp8) rc = launch_moe_cb<BF16, true>(a, cb, max_tasks, inline_align, ws.obuf, s);
         else if (x_kind == MLK_F16) rc = launch_moe_cb<F16, false>(a, cb, max_tasks, inline_align, ws.obuf, s);

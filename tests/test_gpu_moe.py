@@ -204,6 +204,22 @@ def test_fused_moe_single_token(mlk, dtype, fp8, E, K, H, I):
     assert_close(y1, y2.double().cpu().numpy(), RTOL, ATOL, "single-token kernels vs grouped kernels")
 
 
+@pytest.mark.parametrize("slices", [2, 4])
+@pytest.mark.parametrize("T,E,K,fp8", [(3, 8, 2, False), (16, 16, 8, False), (9, 8, 2, True)])
+def test_fused_moe_decode_k_sliced_down(mlk, slices, T, E, K, fp8):
+    """Up to 16 tokens the down projection may slice K across workgroups (the last one to arrive folds
+    the slices in slice order): same result to tolerance, identical from call to call."""
+    from muxi_native_layout_kernels_amd import _lib
+    lib = _lib.load()
+    lib.mlk_set_tunable(7, slices)
+    try:
+        y1 = _moe_case(mlk, T, E, K, 256, 384, torch.bfloat16, 700 + T, fp8=fp8)
+        y2 = _moe_case(mlk, T, E, K, 256, 384, torch.bfloat16, 700 + T, fp8=fp8)
+    finally:
+        lib.mlk_set_tunable(7, 0)
+    assert torch.equal(y1, y2)
+
+
 def test_fused_moe_single_token_expert_map(mlk):
     """A routed expert that is not held locally contributes nothing."""
     from muxi_native_layout_kernels_amd.moe_planC import fused_moe
