@@ -139,6 +139,16 @@ __device__ __forceinline__ float scale_at(const ScaleRow &s, int kblock /* wave-
     return __int_as_float((hi & 2) ? up : lo);
 }
 
+// Wait states between the last MFMA of a block and the first read of its accumulators.  The
+// compiler pads this hazard along the fall-through path; when a taken branch follows the MFMA
+// block directly, a v_accvgpr_read has been observed to run too early and return the previous
+// value of the register (16 wait states cover the 8-pass 16x16x32 instructions).
+__device__ __forceinline__ void mfma_settle() {
+    __builtin_amdgcn_sched_barrier(0);
+    asm volatile("s_nop 7\n\ts_nop 7");
+    __builtin_amdgcn_sched_barrier(0);
+}
+
 // 64-lane xor shuffle of an fp32 through the LDS crossbar (no LDS memory used).
 __device__ __forceinline__ float lane_xor(float v, int mask) {
     int lane = __lane_id();

@@ -239,6 +239,7 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel
         }
 
     }
+    mfma_settle();
 
     constexpr int NTILE = R * CB;
     const int row_tiles = gridDim.x / p.SK;

@@ -485,6 +485,7 @@ __global__ void __launch_bounds__(max_threads_for_tiles(2 * P * CB)) moe_gate_up
             if (u < nt) consume(u);
     }
 
+    mfma_settle();
     // fold the waves in wave order, then SiLU(gate) * up and the layout-B store
     constexpr int NT = R * CB;
 #pragma unroll
@@ -637,6 +638,7 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
                 if (u < nt) consume(u);
         }
 
+        mfma_settle();
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
@@ -940,7 +942,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_tile_kernel(MoeArgs p) {
     for (int r = 0; r < R; ++r)
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
-    TileLoop<T, FP8, CB, R>::run(acc, abase, srow, bs, 0, p.H >> 5, tile_win, blockIdx.x + 7 * task);
+    TileLoop<T, FP8, CB, R>::run(acc, abase, srow, bs, 0, p.H >> 5, tile_win, blockIdx.x + 7 * task, tk.nblocks);
 #pragma unroll
     for (int pr = 0; pr < P; ++pr)
 #pragma unroll
@@ -993,7 +995,7 @@ __global__ void __launch_bounds__(256) moe_down_tile_kernel(MoeArgs p, float *__
         for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
     const int tiles_per = (p.I >> 5) / gridDim.z;          // host: a whole number of windows
     TileLoop<T, FP8, CB, R>::run(acc, abase, srow, bs, blockIdx.z * tiles_per, (blockIdx.z + 1) * tiles_per, tile_win,
-                                 blockIdx.x + 7 * task);
+                                 blockIdx.x + 7 * task, tk.nblocks);
 #pragma unroll
     for (int cb = 0; cb < CB; ++cb) {
         if (cb >= tk.nblocks) continue;

@@ -61,10 +61,12 @@ struct TileBSource {
 
 template <class T, bool FP8, int CB, int R>
 struct TileLoop {
-    // acc[r][cb] += W[stream r][tiles tbeg..tend) . activations ; (tend - tbeg) % KW == 0
+    // acc[r][cb] += W[stream r][tiles tbeg..tend) . activations ; (tend - tbeg) % KW == 0.
+    // Only the first `nb` (workgroup-uniform, 1..CB) token blocks are multiplied; the window is always
+    // fetched whole.
     __device__ static __forceinline__ void run(f32x4 (&acc)[R][CB], const uint8_t *const (&abase)[R],
                                                const ScaleRow (&srow)[R], const TileBSource<CB> &bs, int tbeg,
-                                               int tend, u32x4 *win, int rot_seed) {
+                                               int tend, u32x4 *win, int rot_seed, int nb = CB) {
         constexpr int KW = tile_kw<CB>();
         constexpr int NG = tile_granules_per_thread<CB>();
         constexpr int WG = tile_window_granules<CB>();
@@ -132,15 +134,18 @@ struct TileLoop {
             if (do_stage) stage_load();
 #pragma unroll
             for (int w = 0; w < KW; ++w) {
-                u32x4 b[CB], a[R];
-#pragma unroll
-                for (int cb = 0; cb < CB; ++cb) b[cb] = win[slot * WG + (w * CB + cb) * 68 + q * 17 + r16];
+                u32x4 a[R];
                 weight_operands<FP8, R>(a, wf[slot][w], sc[slot][w]);
 #pragma unroll
-                for (int r = 0; r < R; ++r)
+                for (int cb = 0; cb < CB; ++cb) {
+                    if (cb < nb) {                       // uniform: a scalar branch
+                        const u32x4 b = win[slot * WG + (w * CB + cb) * 68 + q * 17 + r16];
 #pragma unroll
-                    for (int cb = 0; cb < CB; ++cb) acc[r][cb] = T::mfma(a[r], b[cb], acc[r][cb]);
+                        for (int r = 0; r < R; ++r) acc[r][cb] = T::mfma(a[r], b, acc[r][cb]);
+                    }
+                }
             }
+            mfma_settle();
             if (do_issue) issue_a(slot);
             __builtin_amdgcn_sched_barrier(0);
             if (do_stage) stage_store(slot ^ 1);
