@@ -137,6 +137,9 @@ int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k
  *                of each k window through LDS (p2 is ignored); falls back to kernel 1 for a
  *                shape it does not tile (N/16 not a multiple of 4 p1, or K/32 not a multiple
  *                of 4 p3)
+ *   kernel_id 12, 14, 16, 18  kernel 1 with 2, 4, 6 or 8 k tiles in flight per wave instead of the
+ *                default depth; honoured for up to 16 tokens with row-major B and C, otherwise
+ *                the same as kernel 1
  *   p1 = row groups per wave (1, 2 or 4); p3 = K splits across workgroups (>= 1; > 1 needs
  *   `workspace`).
  * workspace: device scratch of at least mlk_gemm_workspace_bytes() bytes, only

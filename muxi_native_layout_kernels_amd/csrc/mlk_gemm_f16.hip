@@ -1,0 +1,6 @@
+// Narrow GeMM kernels instantiated for fp16 weights and activations.
+#include "mlk_gemm_kernels.cuh"
+
+namespace mlk {
+template int launch_modes<F16, false>(const GemmArgs &, int, int, int, int, int, hipStream_t);
+}

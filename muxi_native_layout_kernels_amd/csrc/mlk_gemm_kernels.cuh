@@ -1,0 +1,502 @@
+// Narrow GeMM (1 <= M <= 64 per weight pass) over layout-A weights with
+// v_mfma_f32_16x16x32: C[M, N] = alpha * B[M, K] . A^T + bias.
+//
+// Work decomposition.  A workgroup owns R consecutive row groups (16 R weight
+// rows) and one of SK slices of K.  Its WK waves take the slice's 32-wide k
+// tiles round-robin.  For every k tile a wave loads R weight fragments (1 KiB
+// each, 16 bytes per lane, coalesced, non-temporal) and CB activation
+// fragments (CB = ceil(M/16) <= 4) and issues R*CB MFMAs, so each activation
+// fragment is reused R times and each weight fragment CB times; weights are
+// read from HBM exactly once.  Fragments are prefetched U tiles ahead in a
+// register ring.  Wave partials are folded through LDS in wave order; with
+// SK > 1 workgroup partials go to an fp32 workspace and the last workgroup to
+// arrive for a row tile folds them in slice order, so results are
+// deterministic and never depend on atomics in the data path.
+//
+// The same kernel serves the three operand placements of the reference:
+// row-major or layout-B activations, row-major or layout-C output.  Because
+// the accumulation order is identical, layout-C output followed by the
+// layout-C -> row-major permutation equals the row-major output bit for bit.
+//
+// (template code shared by the per-type translation units mlk_gemm_f16.hip, mlk_gemm_bf16.hip and
+// mlk_gemm_fp8.hip, which instantiate launch_modes<> so that they compile in parallel)
+//
+// Algorithmic traffic per call: N*K*sizeof(W) (+ scales) + M*K*2 + M*N*2 bytes.
+#pragma once
+
+#include "mlk_tile.cuh"
+
+namespace mlk {
+
+
+
+struct GemmArgs {
+    const uint8_t *A;
+    const uint16_t *B;
+    uint16_t *C;
+    const uint16_t *bias;
+    const float *scale;
+    float *partial;      // [SK][row_tiles][R*CB][64] x 4 floats
+    int *counters;       // [row_tiles], zero between calls
+    int M;               // tokens handled by this launch (columns cb0*16 .. )
+    int M_total;         // tokens in the whole problem (row count of B / C)
+    int cb0;             // first 16-token block of this launch
+    int N, K;
+    int WK, SK;
+    int depth;           // 0 = default ring depth, else 2, 4, 6 or 8 (used when one token block is in flight)
+    int rotate;
+    float alpha;
+};
+
+template <class T, bool FP8, int CB, int R, int BMODE, int CMODE, int U, bool STAGE>
+__global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel(GemmArgs p) {
+    extern __shared__ f32x4 red[];  // [WK][R*CB][64]; the staged variant first uses it for two activation windows
+    __shared__ int s_last;
+
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, kept scalar
+    const int q = lane >> 4, r16 = lane & 15;
+    const int sk = blockIdx.x % p.SK;
+    const int rt = blockIdx.x / p.SK;
+    const int rg0 = rt * R;
+    const int tiles_total = p.K >> 5;
+    const int tiles_per = (tiles_total + p.SK - 1) / p.SK;
+    const int tbeg = sk * tiles_per;
+    const int tend = min(tiles_total, tbeg + tiles_per);
+    const int mb_total = (p.M_total + 15) >> 4;
+    const int scale_cols = (p.K + 127) >> 7;
+    constexpr int WBYTES = FP8 ? 1 : 2;
+
+    const uint8_t *abase[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) abase[r] = p.A + (size_t)(rg0 + r) * p.K * 16 * WBYTES;
+
+    // activation fragment source for this lane
+    // Lanes whose token does not exist read the last real token instead: column c of the
+    // product depends only on column c of the activations, and those columns are never stored.
+    const uint16_t *bptr[CB];
+#pragma unroll
+    for (int cb = 0; cb < CB; ++cb) {
+        if (BMODE == MLK_B_NATIVE) {
+            bptr[cb] = p.B + ((size_t)(p.cb0 + cb) * 64 + lane) * 8;
+        } else {
+            int tok = min((p.cb0 + cb) * 16 + r16, p.M_total - 1);
+            bptr[cb] = p.B + (size_t)tok * p.K + q * 8;
+        }
+    }
+    const size_t bstep = (BMODE == MLK_B_NATIVE) ? (size_t)mb_total * 512 : 32;  // elements per k tile
+
+    // the R row groups of a wave (R divides 8, rg0 is a multiple of R) share one row of block scales
+    ScaleRow srow;
+    if (FP8) srow = load_scale_row(p.scale ? p.scale + (size_t)(rg0 >> 3) * scale_cols : nullptr, scale_cols, lane);
+
+    f32x4 acc[R][CB];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    const int nt = (tbeg + wave < tend) ? (tend - tbeg - wave + p.WK - 1) / p.WK : 0;
+
+    WeightFrag<FP8> wf[U][R];
+    u32x4 bf[U][CB];
+    float sc[U];        // one block scale per k tile: the R row groups of a wave share a 128-row block
+    auto issue = [&](int slot, int kt) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
+        if (FP8) sc[slot] = scale_at(srow, kt >> 2);
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * bstep);
+    };
+    auto consume = [&](int slot) {
+        u32x4 a[R], b[CB];
+        float sv[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) sv[r] = FP8 ? sc[slot] : 1.f;
+        weight_operands<FP8, R>(a, wf[slot], sv);
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) b[cb] = bf[slot][cb];
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) acc[r][cb] = T::mfma(a[r], b[cb], acc[r][cb]);
+    };
+    if constexpr (STAGE) {
+        // Row-major activations, staged: in step j the WK waves work on the window of WK
+        // consecutive k tiles [tbeg + w*WK, +WK).  The workgroup fetches the window's
+        // activations with row-contiguous 16-byte loads (WK*64 bytes per token), one step
+        // ahead, and leaves them in LDS in MFMA fragment order (two buffers, one barrier per
+        // step); each wave then reads its own tile's fragments with ds_read_b128.  Fragment
+        // rows are padded (68 granules per tile, 17 per k-octet) against bank conflicts.
+        u32x4 *win = reinterpret_cast<u32x4 *>(red);
+        const int win_granules = p.WK * CB * 68;
+        const int nwin = (tend - tbeg) / p.WK;            // exact: the host only stages when WK divides the slice
+        const int cols = p.WK * 4;                        // 16-byte granules per token in a window
+        const int sh = __builtin_ctz(cols);
+        int rot = (nwin > 0 && p.rotate) ? (int)(((unsigned)rt * 2654435761u >> 7) % (unsigned)nwin) : 0;
+        int w_stage = rot, w_issue = rot;
+        auto advance = [&](int &w) {
+            int cur = w;
+            w = (w + 1 == nwin) ? 0 : w + 1;
+            return cur;
+        };
+        u32x4 breg[CB];
+        auto stage_load = [&]() {
+            const int tile0 = tbeg + advance(w_stage) * p.WK;
+#pragma unroll
+            for (int i = 0; i < CB; ++i) {
+                const int g = threadIdx.x + i * blockDim.x;
+                const int row = g >> sh, colg = g & (cols - 1);
+                const int tok = min(p.cb0 * 16 + row, p.M_total - 1);
+                breg[i] = ld_global_u32x4(p.B + (size_t)tok * p.K + (size_t)tile0 * 32 + colg * 8);
+            }
+        };
+        auto stage_store = [&](int buf) {
+#pragma unroll
+            for (int i = 0; i < CB; ++i) {
+                const int g = threadIdx.x + i * blockDim.x;
+                const int row = g >> sh, colg = g & (cols - 1);
+                win[buf * win_granules + ((colg >> 2) * CB + (row >> 4)) * 68 + (colg & 3) * 17 + (row & 15)] = breg[i];
+            }
+        };
+        auto issue_a = [&](int slot) {
+            const int kt = tbeg + advance(w_issue) * p.WK + wave;
+#pragma unroll
+            for (int r = 0; r < R; ++r) wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
+            if (FP8) sc[slot] = scale_at(srow, kt >> 2);
+        };
+        auto step = [&](int slot, int buf, bool do_stage, bool do_issue) {
+            if (do_stage) stage_load();
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = win[buf * win_granules + (wave * CB + cb) * 68 + q * 17 + r16];
+            consume(slot);
+            if (do_issue) issue_a(slot);
+            __builtin_amdgcn_sched_barrier(0);
+            if (do_stage) stage_store(buf ^ 1);
+            __syncthreads();
+        };
+        static_assert(U % 2 == 0, "the staged loop alternates two LDS buffers inside a U-step unroll");
+        if (nwin > 0) {
+            stage_load();
+            stage_store(0);
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < nwin) issue_a(u);
+            __syncthreads();
+            int j = 0;
+            for (; j + 2 * U <= nwin; j += U) {
+#pragma unroll
+                for (int u = 0; u < U; ++u) step(u, u & 1, true, true);
+            }
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (j + u < nwin) step(u, u & 1, j + u + 1 < nwin, j + u + U < nwin);
+            j += U;
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (j + u < nwin) step(u, u & 1, j + u + 1 < nwin, false);
+        }
+        __syncthreads();   // the windows are dead; the same LDS now serves the wave fold
+    } else {
+        // The wave visits its k tiles in a rotated order that differs from row tile to row tile:
+        // workgroups that run side by side then read different parts of the (small, shared)
+        // activation matrix at any moment instead of all hitting the same cache lines.
+        int jcur = (nt > 0 && p.rotate) ? (int)(((unsigned)rt * 2654435761u >> 7) % (unsigned)nt) : 0;
+        auto next_tile = [&]() {
+            int t = tbeg + wave + jcur * p.WK;
+            jcur = (jcur + 1 == nt) ? 0 : jcur + 1;
+            return t;
+        };
+
+        // Register ring of U k-tiles; the steady-state loop is branch-free so the loads stay
+        // U tiles deep in flight.
+        if (nt >= U) {
+    #pragma unroll
+            for (int u = 0; u < U; ++u) issue(u, next_tile());
+            int i = 0;
+            for (; i + 2 * U <= nt; i += U) {
+    #pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    consume(u);
+                    issue(u, next_tile());
+                    __builtin_amdgcn_sched_barrier(0);  // keep each refill right behind its consume
+                }
+            }
+            const int rem = nt - i - U;
+    #pragma unroll
+            for (int u = 0; u < U; ++u) {
+                consume(u);
+                if (u < rem) issue(u, next_tile());
+            }
+    #pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < rem) consume(u);
+        } else {
+    #pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < nt) issue(u, next_tile());
+    #pragma unroll
+            for (int u = 0; u < U; ++u)
+                if (u < nt) consume(u);
+        }
+
+    }
+    mfma_settle();
+
+    constexpr int NTILE = R * CB;
+    const int row_tiles = gridDim.x / p.SK;
+
+    auto epilogue = [&](int j, f32x4 v) {
+        const int r = j / CB, cb = j - r * CB;
+        const int n = (rg0 + r) * 16 + 4 * q;
+        const int tok = (p.cb0 + cb) * 16 + r16;
+        if (tok >= p.M_total) return;
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o[i] = p.alpha * v[i];
+            if (p.bias) o[i] += T::to_f32(p.bias[n + i]);
+        }
+        size_t off;
+        if (CMODE == MLK_C_NATIVE)
+            off = ((((size_t)(n >> 5) * mb_total + (tok >> 4)) * 4 + ((n & 31) >> 3)) * 16 + (tok & 15)) * 8 + (n & 7);
+        else
+            off = (size_t)tok * p.N + n;
+        store4<T>(p.C + off, o[0], o[1], o[2], o[3]);
+    };
+    f32x4 *part = reinterpret_cast<f32x4 *>(p.partial);
+    auto part_at = [&](int s, int j) -> size_t { return (((size_t)s * row_tiles + rt) * NTILE + j) * 64 + lane; };
+
+    if (p.WK == 1) {
+        // a single wave: tiles stay in registers
+        if (p.SK == 1) {
+#pragma unroll
+            for (int r = 0; r < R; ++r)
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb) epilogue(r * CB + cb, acc[r][cb]);
+            return;
+        }
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) st_agent_f32x4(&part[part_at(sk, r * CB + cb)], acc[r][cb]);
+    } else {
+        // fold the WK waves through LDS in wave order; wave w then owns tiles j = w, w + WK, ...
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) red[(wave * NTILE + r * CB + cb) * 64 + lane] = acc[r][cb];
+        __syncthreads();
+        for (int j = wave; j < NTILE; j += p.WK) {
+            f32x4 v = red[j * 64 + lane];
+            for (int w = 1; w < p.WK; ++w) v += red[(w * NTILE + j) * 64 + lane];
+            if (p.SK == 1) epilogue(j, v);
+            else st_agent_f32x4(&part[part_at(sk, j)], v);
+        }
+        if (p.SK == 1) return;
+    }
+
+    // ---- K split across workgroups: the partial is published with agent-coherent stores, the
+    // last workgroup to arrive for this row tile folds all slices in slice order.  Every wave
+    // waits for its own stores to be acknowledged before the barrier; the arrival counter is
+    // bumped after the barrier, so a workgroup that sees SK-1 earlier arrivals can read all
+    // partials.
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int prev = __hip_atomic_fetch_add(&p.counters[rt], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (prev == p.SK - 1);
+        if (s_last) __hip_atomic_store(&p.counters[rt], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last) return;
+    for (int j = wave; j < NTILE; j += p.WK) {
+        f32x4 v = {0.f, 0.f, 0.f, 0.f};
+        for (int s = 0; s < p.SK; ++s) v += ld_agent_f32x4(&part[part_at(s, j)]);
+        epilogue(j, v);
+    }
+}
+
+// Kernel 2: row-shared tile kernel (see mlk_tile.cuh).  Four waves per workgroup, R row groups
+// per wave, activations of every k window staged once per workgroup in LDS; K is split across
+// workgroups only (SK), folded by the last workgroup to arrive with agent-coherent loads.
+template <class T, bool FP8, int CB, int R, int BMODE, int CMODE>
+__global__ void __launch_bounds__(256) gemm_tile_kernel(GemmArgs p) {
+    extern __shared__ u32x4 tile_win[];
+    __shared__ int s_last;
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int q = lane >> 4, r16 = lane & 15;
+    const int sk = blockIdx.x % p.SK;
+    const int rt = blockIdx.x / p.SK;
+    const int rg0 = (rt * kTileWaves + wave) * R;
+    const int tiles_total = p.K >> 5;
+    const int tiles_per = tiles_total / p.SK;          // host: a whole number of windows
+    const int tbeg = sk * tiles_per, tend = tbeg + tiles_per;
+    const int mb_total = (p.M_total + 15) >> 4;
+    const int scale_cols = (p.K + 127) >> 7;
+    constexpr int WBYTES = FP8 ? 1 : 2;
+
+    const uint8_t *abase[R];
+    ScaleRow srow[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        abase[r] = p.A + (size_t)(rg0 + r) * p.K * 16 * WBYTES;
+        if (FP8)
+            srow[r] = load_scale_row(p.scale ? p.scale + (size_t)((rg0 + r) >> 3) * scale_cols : nullptr, scale_cols, lane);
+    }
+    TileBSource<CB> bs;
+    bs.native_token_major = false;
+    if (BMODE == MLK_B_NATIVE) {
+        bs.native_tile_stride = (size_t)mb_total * 512;
+        bs.row[0] = p.B + (size_t)p.cb0 * 512;
+    } else {
+        bs.native_tile_stride = 0;
+#pragma unroll
+        for (int i = 0; i < tile_granules_per_thread<CB>(); ++i) {
+            int block, token, colg;
+            tile_row_of<CB>(i, threadIdx.x, block, token, colg);
+            const int tok = min((p.cb0 + block) * 16 + token, p.M_total - 1);
+            bs.row[i] = p.B + (size_t)tok * p.K + colg * 8;
+        }
+    }
+    f32x4 acc[R][CB];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    TileLoop<T, FP8, CB, R>::run(acc, abase, srow, bs, tbeg, tend, tile_win, p.rotate ? rt : 0);
+
+    constexpr int NTILE = R * CB;
+    const int row_tiles = gridDim.x / p.SK;
+    auto epilogue = [&](int r, int cb, f32x4 v) {
+        const int n = (rg0 + r) * 16 + 4 * q;
+        const int tok = (p.cb0 + cb) * 16 + r16;
+        if (tok >= p.M_total) return;
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o[i] = p.alpha * v[i];
+            if (p.bias) o[i] += T::to_f32(p.bias[n + i]);
+        }
+        size_t off;
+        if (CMODE == MLK_C_NATIVE)
+            off = ((((size_t)(n >> 5) * mb_total + (tok >> 4)) * 4 + ((n & 31) >> 3)) * 16 + (tok & 15)) * 8 + (n & 7);
+        else
+            off = (size_t)tok * p.N + n;
+        store4<T>(p.C + off, o[0], o[1], o[2], o[3]);
+    };
+    if (p.SK == 1) {
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+            for (int cb = 0; cb < CB; ++cb) epilogue(r, cb, acc[r][cb]);
+        return;
+    }
+    f32x4 *part = reinterpret_cast<f32x4 *>(p.partial);
+    auto part_at = [&](int s, int j) -> size_t {
+        return ((((size_t)s * row_tiles + rt) * kTileWaves + wave) * NTILE + j) * 64 + lane;
+    };
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) st_agent_f32x4(&part[part_at(sk, r * CB + cb)], acc[r][cb]);
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int prev = __hip_atomic_fetch_add(&p.counters[rt], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        s_last = (prev == p.SK - 1);
+        if (s_last) __hip_atomic_store(&p.counters[rt], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!s_last) return;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int cb = 0; cb < CB; ++cb) {
+            f32x4 v = {0.f, 0.f, 0.f, 0.f};
+            for (int s = 0; s < p.SK; ++s) v += ld_agent_f32x4(&part[part_at(s, r * CB + cb)]);
+            epilogue(r, cb, v);
+        }
+}
+
+// Can kernel 2 run this problem with these parameters?
+static bool tile_kernel_fits(const GemmArgs &p, int R) {
+    const int tiles_total = p.K / 32;
+    return (p.N / 16) % (kTileWaves * R) == 0 && p.SK >= 1 && tiles_total % (p.SK * kTileKW) == 0;  // CB <= 4 here
+}
+
+template <class T, bool FP8, int CB, int R, int BMODE, int CMODE>
+static int launch_tile(const GemmArgs &p, hipStream_t s) {
+    int row_tiles = (p.N / 16) / (kTileWaves * R);
+    gemm_tile_kernel<T, FP8, CB, R, BMODE, CMODE><<<row_tiles * p.SK, 256, tile_lds_bytes<CB>(), s>>>(p);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+template <class T, bool FP8, int CB, int R, int BMODE, int CMODE>
+static int launch(const GemmArgs &p, hipStream_t s) {
+    constexpr int U = (R * CB >= 8) ? 2 : ((R * CB >= 4) ? 3 : 4);
+    GemmArgs q = p;
+    while (q.WK * 64 > max_threads_for_tiles(R * CB) || (size_t)q.WK * R * CB * 1024 > 64 * 1024) q.WK >>= 1;
+    int row_tiles = (q.N / 16) / R;
+    int grid = row_tiles * q.SK;
+    size_t lds = q.WK > 1 ? (size_t)q.WK * R * CB * 1024 : 0;
+    if constexpr (BMODE == MLK_B_ROWMAJOR) {
+        // stage row-major activations through LDS when every K slice is a whole number of WK-tile windows
+        const int tiles_total = q.K / 32;
+        const int tiles_per = (tiles_total + q.SK - 1) / q.SK;
+        const size_t win_bytes = (size_t)2 * q.WK * CB * 68 * 16;
+        // (measured: staging pays only from three token blocks up; below that the direct gather wins)
+        if (g_tunable[1] && CB >= 3 && q.WK >= 2 && tiles_total % q.SK == 0 && tiles_per % q.WK == 0 && win_bytes <= 48 * 1024) {
+            constexpr int US = (R * CB >= 8) ? 2 : 4;
+            if (win_bytes > lds) lds = win_bytes;
+            gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, US, true><<<grid, q.WK * 64, lds, s>>>(q);
+            MLK_LAUNCH_CHECK();
+            return MLK_OK;
+        }
+    }
+    if constexpr (CB == 1 && BMODE == MLK_B_ROWMAJOR && CMODE == MLK_C_ROWMAJOR) {
+        // kernel ids 12, 14, 16, 18: explicit depth of the register ring (k tiles in flight per wave)
+#define MLK_DEPTH(UU)                                                                                   \
+    if (q.depth == UU) {                                                                                \
+        gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, UU, false><<<grid, q.WK * 64, lds, s>>>(q);       \
+        MLK_LAUNCH_CHECK();                                                                             \
+        return MLK_OK;                                                                                  \
+    }
+        MLK_DEPTH(2) MLK_DEPTH(4) MLK_DEPTH(6) MLK_DEPTH(8)
+#undef MLK_DEPTH
+    }
+    gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, U, false><<<grid, q.WK * 64, lds, s>>>(q);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+template <class T, bool FP8, int BMODE, int CMODE>
+static int launch_rc(const GemmArgs &p, int kernel_id, int R, int CB, hipStream_t s) {
+#define MLK_CASE(RR, CC)                                                                        \
+    if (R == RR && CB == CC)                                                                    \
+        return (kernel_id == 2 && tile_kernel_fits(p, RR)) ? launch_tile<T, FP8, CC, RR, BMODE, CMODE>(p, s) \
+                                                          : launch<T, FP8, CC, RR, BMODE, CMODE>(p, s);
+    MLK_CASE(1, 1) MLK_CASE(1, 2) MLK_CASE(1, 3) MLK_CASE(1, 4)
+    MLK_CASE(2, 1) MLK_CASE(2, 2) MLK_CASE(2, 3) MLK_CASE(2, 4)
+    MLK_CASE(4, 1) MLK_CASE(4, 2) MLK_CASE(4, 3) MLK_CASE(4, 4)
+#undef MLK_CASE
+    return fail(MLK_ERR_INVALID, "gemm: unsupported (row groups per wave, column blocks)");
+}
+
+template <class T, bool FP8>
+int launch_modes(const GemmArgs &p, int kernel_id, int b_mode, int c_mode, int R, int CB, hipStream_t s) {
+    if (b_mode == MLK_B_ROWMAJOR && c_mode == MLK_C_ROWMAJOR)
+        return launch_rc<T, FP8, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR>(p, kernel_id, R, CB, s);
+    if (!FP8) {
+        if (b_mode == MLK_B_NATIVE && c_mode == MLK_C_ROWMAJOR)
+            return launch_rc<T, false, MLK_B_NATIVE, MLK_C_ROWMAJOR>(p, kernel_id, R, CB, s);
+        if (b_mode == MLK_B_NATIVE && c_mode == MLK_C_NATIVE)
+            return launch_rc<T, false, MLK_B_NATIVE, MLK_C_NATIVE>(p, kernel_id, R, CB, s);
+    }
+    return fail(MLK_ERR_INVALID, "gemm: unsupported operand placement");
+}
+
+}  // namespace mlk

@@ -138,6 +138,10 @@ def scan_gemm(table, shapes, tokens, iters):
             # kernel 2 (row-shared tiles): 4 waves x p1 row groups per workgroup, K split only across workgroups
             grid += [(2, r, 1, sk) for r in (1, 2, 4) for sk in (1, 2, 4, 8)
                      if (n // 16) % (4 * r) == 0 and (k // 32) % (4 * sk) == 0 and m > 16]
+            # kernels 12..18: the wave kernel with 2, 4, 6 or 8 k tiles in flight per wave (one token block,
+            # row-major activations and output)
+            if m <= 16 and mode in ("rowmajor", "fp8"):
+                grid += [(10 + u, r, w, sk) for (_, r, w, sk) in list(grid) if _ == 1 for u in (2, 4, 6, 8)]
             for kid, p1, p2, p3 in grid:
                 if (n // 16) % p1:
                     continue

@@ -85,6 +85,34 @@ def test_gemm_tile_kernel_soft_fp8(mlk):
     assert_close(c, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), b), RTOL, ATOL, "tile fp8")
 
 
+@pytest.mark.parametrize("kid", [12, 14, 16, 18])
+@pytest.mark.parametrize("p1,p2,p3", [(1, 1, 1), (4, 2, 1), (2, 8, 2), (1, 16, 1)])
+@pytest.mark.parametrize("m", [1, 7, 16, 40])
+def test_gemm_ring_depth_kernel_ids(mlk, kid, p1, p2, p3, m):
+    """kernelId 12..18: kernel 1 with 2..8 k tiles in flight per wave.  The summation order does not depend
+    on the depth, so the result is bit-equal to kernel 1's; above 16 tokens the ids mean kernel 1."""
+    n, k = 512, 1024 + 32 * 5                    # 37 k tiles: fewer than, equal to and more than the ring at some split
+    w = randn((n, k), torch.float16, 0.02, 31)
+    b = randn((m, k), torch.float16, 1.0, 32)
+    a = pack_a(w).cuda()
+    c = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, kernelParam1=p1, kernelParam2=p2, kernelParam3=p3, kernelId=kid)
+    assert_close(c, ogemm.linear_expected(w, b), RTOL, ATOL, "ring depth id %d" % kid)
+    c1 = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, kernelParam1=p1, kernelParam2=p2, kernelParam3=p3, kernelId=1)
+    assert torch.equal(c, c1)
+
+
+def test_gemm_ring_depth_soft_fp8(mlk):
+    n, k, m = 512, 1024, 9
+    codes = fp8_codes((n, k), 41)
+    b = randn((m, k), torch.bfloat16, 1.0, 42)
+    g = torch.Generator().manual_seed(43)
+    scale = (torch.rand((n // 128, k // 128), generator=g) * 0.02 + 0.001).float()
+    for kid in (12, 14, 16, 18):
+        c = mlk.gemm_layoutA_soft_fp8_wapper(pack_a(codes).cuda(), scale.cuda(), b.cuda(), n, m, k, kernelParam1=2,
+                                             kernelParam2=4, kernelParam3=1, kernelId=kid)
+        assert_close(c, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), b), RTOL, ATOL, "fp8 depth")
+
+
 def test_gemm_special_cases(mlk):
     n = k = 256
     eye = torch.eye(n, dtype=torch.float16)
