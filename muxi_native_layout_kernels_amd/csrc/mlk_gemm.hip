@@ -42,7 +42,7 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
     MLK_REQUIRE(kernel_id == 1 || kernel_id == 2 || kernel_id == 12 || kernel_id == 14 || kernel_id == 16 ||
                     kernel_id == 18,
                 "gemm: unknown kernel id");
-    MLK_REQUIRE(p1 == 1 || p1 == 2 || p1 == 4, "gemm: row groups per wave (p1) must be 1, 2 or 4");
+    MLK_REQUIRE(p1 == 1 || p1 == 2 || p1 == 4 || p1 == 8, "gemm: row groups per wave (p1) must be 1, 2, 4 or 8");
     MLK_REQUIRE((n / 16) % p1 == 0, "gemm: row groups per wave (p1) must divide N/16");
     MLK_REQUIRE(p2 == 1 || p2 == 2 || p2 == 4 || p2 == 8 || p2 == 16, "gemm: waves per workgroup (p2) must be 1, 2, 4, 8 or 16");
     MLK_REQUIRE(p3 >= 1 && p3 <= 64, "gemm: K splits across workgroups (p3) must be 1..64");
@@ -96,10 +96,11 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
         g.M = mm;
         g.cb0 = c0 / 16;
         int cb = (mm + 15) / 16;
+        const int r = (p1 == 8 && cb > 1) ? 4 : p1;   // eight row groups per wave exist for one token block only
         int rc;
-        if (fp8) rc = launch_modes<BF16, true>(g, kernel_id, b_mode, c_mode, p1, cb, s);
-        else if (x_kind == MLK_F16) rc = launch_modes<F16, false>(g, kernel_id, b_mode, c_mode, p1, cb, s);
-        else rc = launch_modes<BF16, false>(g, kernel_id, b_mode, c_mode, p1, cb, s);
+        if (fp8) rc = launch_modes<BF16, true>(g, kernel_id, b_mode, c_mode, r, cb, s);
+        else if (x_kind == MLK_F16) rc = launch_modes<F16, false>(g, kernel_id, b_mode, c_mode, r, cb, s);
+        else rc = launch_modes<BF16, false>(g, kernel_id, b_mode, c_mode, r, cb, s);
         if (rc != MLK_OK) return rc;
     }
     return MLK_OK;

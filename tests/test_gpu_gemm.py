@@ -86,7 +86,7 @@ def test_gemm_tile_kernel_soft_fp8(mlk):
 
 
 @pytest.mark.parametrize("kid", [12, 14, 16, 18])
-@pytest.mark.parametrize("p1,p2,p3", [(1, 1, 1), (4, 2, 1), (2, 8, 2), (1, 16, 1)])
+@pytest.mark.parametrize("p1,p2,p3", [(1, 1, 1), (4, 2, 1), (2, 8, 2), (1, 16, 1), (8, 4, 1), (8, 2, 2)])
 @pytest.mark.parametrize("m", [1, 7, 16, 40])
 def test_gemm_ring_depth_kernel_ids(mlk, kid, p1, p2, p3, m):
     """kernelId 12..18: kernel 1 with 2..8 k tiles in flight per wave.  The summation order does not depend
@@ -108,9 +108,10 @@ def test_gemm_ring_depth_soft_fp8(mlk):
     g = torch.Generator().manual_seed(43)
     scale = (torch.rand((n // 128, k // 128), generator=g) * 0.02 + 0.001).float()
     for kid in (12, 14, 16, 18):
-        c = mlk.gemm_layoutA_soft_fp8_wapper(pack_a(codes).cuda(), scale.cuda(), b.cuda(), n, m, k, kernelParam1=2,
-                                             kernelParam2=4, kernelParam3=1, kernelId=kid)
-        assert_close(c, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), b), RTOL, ATOL, "fp8 depth")
+        for p1 in (2, 8):         # eight row groups per wave = one 128-row scale block
+            c = mlk.gemm_layoutA_soft_fp8_wapper(pack_a(codes).cuda(), scale.cuda(), b.cuda(), n, m, k, kernelParam1=p1,
+                                                 kernelParam2=4, kernelParam3=1, kernelId=kid)
+            assert_close(c, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), b), RTOL, ATOL, "fp8 depth")
 
 
 def test_gemm_special_cases(mlk):
