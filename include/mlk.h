@@ -53,7 +53,8 @@ const char *mlk_last_error(void);
  *   id 2, 3  single-token MoE, gate/up kernel: row groups per workgroup and waves splitting K
  *         (defaults 1 and 8; 2 * id2 * id3 <= 16)
  *   id 4  single-token MoE, down kernel: waves per workgroup (default 16)
- *   id 5  single-token MoE: 16-byte loads in flight per wave, 2, 3, 4, 6 or 8 (default 4)
+ *   id 5  single-token MoE: 16-byte loads in flight per wave, 2, 3, 4, 6 or 8 (default 0 = 2 for
+ *         soft-FP8 weights, 4 otherwise)
  *   id 7  decode MoE (2..16 tokens), down kernel: row groups per wave = K slices across
  *         workgroups, 1, 2 or 4 (default 0 = 4 for soft-FP8 weights, 1 otherwise)
  * No counterpart in the reference. */

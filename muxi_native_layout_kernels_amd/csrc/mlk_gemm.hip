@@ -7,8 +7,9 @@ namespace mlk {
 constexpr size_t kCounterBytes = 64 * 1024;
 
 // Experiment switches (mlk_set_tunable): [0] rotate the k-tile order per row tile,
-// [1] stage row-major activations through LDS.
-int g_tunable[8] = {1, 1, 1, 8, 16, 4, 0, 0};
+// [1] stage row-major activations through LDS, [2]..[5] and [7] shape the fused MoE kernels
+// (listed with the declaration of mlk_set_tunable); 0 means automatic for [5] and [7].
+int g_tunable[8] = {1, 1, 1, 8, 16, 0, 0, 0};
 
 extern template int launch_modes<F16, false>(const GemmArgs &, int, int, int, int, int, hipStream_t);
 extern template int launch_modes<BF16, false>(const GemmArgs &, int, int, int, int, int, hipStream_t);

@@ -729,26 +729,26 @@ __device__ __forceinline__ void gemv1_tile(const u32x4 &w, float s, const u32x4 
     }
 }
 
-// The tiles ks, ks + WK, ... of one row group against an activation vector in LDS.  The first
-// weight loads are put in flight, then `stage` runs (the caller copies the activations to LDS and
-// synchronises the workgroup there), then the rest streams; the 16 row sums end in red16[0..15].
+// The nt tiles first, first + step, ... of one row group against an activation vector in LDS
+// (xs is indexed by the absolute tile).  The first weight loads are put in flight, then `stage`
+// runs (the wave copies the activations of its own tiles to LDS; no other wave reads them, so no
+// workgroup barrier is needed), then the rest streams; the 16 row sums end in red16[0..15].
 template <class T, bool FP8, int U, class Stage>
-__device__ __forceinline__ void gemv1_stream(const uint8_t *rowgroup, int tiles, int ks, int WK, const u32x4 *xs,
+__device__ __forceinline__ void gemv1_stream(const uint8_t *rowgroup, int first, int nt, int step, const u32x4 *xs,
                                              const ScaleRow &srow, float *red16, Stage stage) {
     constexpr int TKG = FP8 ? 8 : 4;                 // activation granules (8 elements) per tile
     const int lane = threadIdx.x & 63;
     const int oct = FP8 ? (lane >> 3) : (lane >> 4);
-    const u32x4 *ap = reinterpret_cast<const u32x4 *>(rowgroup) + (size_t)ks * 64 + lane;
-    const int stride = WK * 64;
-    const int nt = ks < tiles ? (tiles - ks + WK - 1) / WK : 0;
+    const u32x4 *ap = reinterpret_cast<const u32x4 *>(rowgroup) + (size_t)first * 64 + lane;
+    const int stride = step * 64;
     float acc[2] = {0.f, 0.f};
     u32x4 buf[U];
     float sc[U];
     auto issue = [&](int u, int j) {
         buf[u] = ld_stream_u32x4(ap + (size_t)j * stride);
-        sc[u] = FP8 ? scale_at(srow, (ks + j * WK) >> 1) : 1.f;
+        sc[u] = FP8 ? scale_at(srow, (first + j * step) >> 1) : 1.f;
     };
-    auto consume = [&](int u, int j) { gemv1_tile<T, FP8>(buf[u], sc[u], xs, (ks + j * WK) * TKG + oct, acc); };
+    auto consume = [&](int u, int j) { gemv1_tile<T, FP8>(buf[u], sc[u], xs, (first + j * step) * TKG + oct, acc); };
     const bool full = nt >= U;
     if (full) {
 #pragma unroll
@@ -801,6 +801,16 @@ __device__ __forceinline__ void gemv1_stream(const uint8_t *rowgroup, int tiles,
     }
 }
 
+// Copy the activation granules of the tiles first, first + step, ... (nt of them) into LDS: the
+// wave's own share of the vector, so the waves of a workgroup never wait for each other.
+template <int TKG>
+__device__ __forceinline__ void gemv1_fill(u32x4 *dst, const u32x4 *src, int first, int nt, int step, int lane) {
+    for (int i = lane; i < nt * TKG; i += 64) {
+        const int idx = (first + (i / TKG) * step) * TKG + (i % TKG);
+        dst[idx] = src[idx];
+    }
+}
+
 struct Moe1Args {
     const uint8_t *W1, *W2;
     const float *S1, *S2;
@@ -835,9 +845,12 @@ __global__ void __launch_bounds__(1024) moe_gate_up_gemv1_kernel(Moe1Args p) {
     ScaleRow srow;
     if (FP8)
         srow = load_scale_row(p.S1 ? p.S1 + ((size_t)e * (2 * p.I >> 7) + (rg >> 3)) * (p.H >> 7) : nullptr, p.H >> 7, lane);
-    gemv1_stream<T, FP8, U>(rowgroup, p.H / TK, ks, p.WK, xs, srow, red[wave], [&]() {
-        for (int i = threadIdx.x; i < (p.H >> 3); i += blockDim.x) xs[i] = reinterpret_cast<const u32x4 *>(p.X)[i];
-        __syncthreads();
+    const int tiles = p.H / TK;
+    const int count = ks < tiles ? (tiles - ks + p.WK - 1) / p.WK : 0;
+    constexpr int TKG = FP8 ? 8 : 4;
+    gemv1_stream<T, FP8, U>(rowgroup, ks, count, p.WK, xs, srow, red[wave], [&]() {
+        // the 2 G waves that share these k tiles each write the same values
+        gemv1_fill<TKG>(xs, reinterpret_cast<const u32x4 *>(p.X), ks, count, p.WK, lane);
     });
     __syncthreads();
     if (threadIdx.x < 16 * p.G) {
@@ -877,12 +890,13 @@ __global__ void __launch_bounds__(1024) moe_down_gemv1_kernel(Moe1Args p) {
     if (FP8)
         srow = load_scale_row(p.S2 ? p.S2 + ((size_t)ee * (p.H >> 7) + (blockIdx.x >> 3)) * (p.I >> 7) : nullptr,
                               p.I >> 7, lane);
-    gemv1_stream<T, FP8, U>(rowgroup, e >= 0 ? p.I / TK : 0, ks, wpt, hs + (size_t)(pair < p.K ? pair : 0) * gran, srow,
-                            red[wave], [&]() {
-                                for (int i = threadIdx.x; i < p.K * gran; i += blockDim.x)
-                                    hs[i] = reinterpret_cast<const u32x4 *>(p.Hd)[i];
-                                __syncthreads();
-                            });
+    const int tiles = p.I / TK;
+    const int count = (e >= 0 && ks < tiles) ? (tiles - ks + wpt - 1) / wpt : 0;
+    constexpr int TKG = FP8 ? 8 : 4;
+    u32x4 *mine = hs + (size_t)(pair < p.K ? pair : 0) * gran;
+    const u32x4 *src = reinterpret_cast<const u32x4 *>(p.Hd) + (size_t)(pair < p.K ? pair : 0) * gran;
+    gemv1_stream<T, FP8, U>(rowgroup, ks, count, wpt, mine, srow, red[wave],
+                            [&]() { gemv1_fill<TKG>(mine, src, ks, count, wpt, lane); });
     __syncthreads();
     if (threadIdx.x < 16) {
         float y = 0.f;
@@ -1285,10 +1299,11 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
     } while (0)
 #define MLK_MOE1_U(TT, F8)                                                          \
     do {                                                                            \
-        if (g_tunable[5] == 2) MLK_MOE1(TT, F8, 2);                                 \
-        else if (g_tunable[5] == 3) MLK_MOE1(TT, F8, 3);                            \
-        else if (g_tunable[5] == 6) MLK_MOE1(TT, F8, 6);                            \
-        else if (g_tunable[5] == 8) MLK_MOE1(TT, F8, 8);                            \
+        const int depth = g_tunable[5] ? g_tunable[5] : (F8 ? 2 : 4);               \
+        if (depth == 2) MLK_MOE1(TT, F8, 2);                                        \
+        else if (depth == 3) MLK_MOE1(TT, F8, 3);                                   \
+        else if (depth == 6) MLK_MOE1(TT, F8, 6);                                   \
+        else if (depth == 8) MLK_MOE1(TT, F8, 8);                                   \
         else MLK_MOE1(TT, F8, 4);                                                   \
     } while (0)
             if (fp8) MLK_MOE1_U(BF16, true);
