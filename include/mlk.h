@@ -141,7 +141,7 @@ int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k
  *   kernel_id 12, 14, 16, 18  kernel 1 with 2, 4, 6 or 8 k tiles in flight per wave instead of the
  *                default depth; honoured for up to 16 tokens with row-major B and C, otherwise
  *                the same as kernel 1
- *   p1 = row groups per wave (1, 2 or 4; 8 is taken for up to 16 tokens and means 4 above);
+ *   p1 = row groups per wave (1, 2, 4 or 8; 8 means 4 when more than 16 tokens meet a native B or C);
  *   p3 = K splits across workgroups (>= 1; > 1 needs
  *   `workspace`).
  * workspace: device scratch of at least mlk_gemm_workspace_bytes() bytes, only

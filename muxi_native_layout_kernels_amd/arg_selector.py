@@ -24,7 +24,7 @@ What the columns select on gfx950 (the rows are produced by the scripts in
                              12, 14, 16, 18 = kernel 1 with 2, 4, 6, 8 k tiles in flight per
                                  wave (up to 16 tokens, row-major activations and output;
                                  otherwise the same as 1)
-                kernelParam1 row groups per wave (1, 2, 4; 8 for up to 16 tokens)
+                kernelParam1 row groups per wave (1, 2, 4, 8)
                 kernelParam2 waves per workgroup splitting K (1..16)
                 kernelParam3 K splits across workgroups
 """

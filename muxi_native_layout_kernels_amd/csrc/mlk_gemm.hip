@@ -97,7 +97,8 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
         g.M = mm;
         g.cb0 = c0 / 16;
         int cb = (mm + 15) / 16;
-        const int r = (p1 == 8 && cb > 1) ? 4 : p1;   // eight row groups per wave exist for one token block only
+        // eight row groups per wave exist for one token block, or with row-major B and C
+        const int r = (p1 == 8 && cb > 1 && !(b_mode == MLK_B_ROWMAJOR && c_mode == MLK_C_ROWMAJOR)) ? 4 : p1;
         int rc;
         if (fp8) rc = launch_modes<BF16, true>(g, kernel_id, b_mode, c_mode, r, cb, s);
         else if (x_kind == MLK_F16) rc = launch_modes<F16, false>(g, kernel_id, b_mode, c_mode, r, cb, s);

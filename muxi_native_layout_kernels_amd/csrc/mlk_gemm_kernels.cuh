@@ -483,8 +483,13 @@ static int launch_rc(const GemmArgs &p, int kernel_id, int R, int CB, hipStream_
     MLK_CASE(2, 1) MLK_CASE(2, 2) MLK_CASE(2, 3) MLK_CASE(2, 4)
     MLK_CASE(4, 1) MLK_CASE(4, 2) MLK_CASE(4, 3) MLK_CASE(4, 4)
 #undef MLK_CASE
-    // eight row groups per wave: one token block, wave kernel only
+    // eight row groups per wave: wave kernel only; more than one token block only with row-major B and C
     if (R == 8 && CB == 1) return launch<T, FP8, 1, 8, BMODE, CMODE>(p, s);
+    if constexpr (BMODE == MLK_B_ROWMAJOR && CMODE == MLK_C_ROWMAJOR) {
+        if (R == 8 && CB == 2) return launch<T, FP8, 2, 8, BMODE, CMODE>(p, s);
+        if (R == 8 && CB == 3) return launch<T, FP8, 3, 8, BMODE, CMODE>(p, s);
+        if (R == 8 && CB == 4) return launch<T, FP8, 4, 8, BMODE, CMODE>(p, s);
+    }
     return fail(MLK_ERR_INVALID, "gemm: unsupported (row groups per wave, column blocks)");
 }
 

@@ -134,8 +134,9 @@ def scan_gemm(table, shapes, tokens, iters):
             want = b.float() @ w0.t()
             b_in = ops.layoutB(b) if mode in ("continuous", "native") else b
             best = None
-            # eight row groups per wave exist for one token block only
-            grid = [(1, r, w, sk) for r in ((1, 2, 4, 8) if m <= 16 else (1, 2, 4)) for w in (1, 2, 4, 8, 16)
+            # eight row groups per wave exist for one token block, or with row-major activations and output
+            grid = [(1, r, w, sk) for r in ((1, 2, 4, 8) if m <= 16 or mode in ("rowmajor", "fp8") else (1, 2, 4))
+                    for w in (1, 2, 4, 8, 16)
                     for sk in ((1, 2, 4) if n <= 8192 else (1,))]
             # kernel 2 (row-shared tiles): 4 waves x p1 row groups per workgroup, K split only across workgroups
             grid += [(2, r, 1, sk) for r in (1, 2, 4) for sk in (1, 2, 4, 8)
