@@ -52,10 +52,17 @@ def _time_graph(calls, iters):
         with torch.cuda.graph(graph, stream=stream):
             for i in range(iters):
                 calls[i % len(calls)]()
+        # The capture leaves the GPU idle and the first replays after an idle period run several percent
+        # below the steady state, so replay un-timed for about 10 ms first, then time back-to-back replays.
         graph.replay()
         torch.cuda.synchronize()
-        # back-to-back replays, timed as a whole: clocks settle lower under a sustained stream of calls than
-        # in a short burst, and the table should hold what wins in steady state
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        for _ in range(max(1, int(10.0 / max(e0.elapsed_time(e1), 0.05)))):
+            graph.replay()
         e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         e0.record()
         for _ in range(3):
