@@ -220,6 +220,20 @@ def test_fused_moe_decode_k_sliced_down(mlk, slices, T, E, K, fp8):
     assert torch.equal(y1, y2)
 
 
+@pytest.mark.parametrize("T,E,K,H,I,fp8", [
+    (1, 4, 1, 128, 128, False),      # one pick: all 16 waves of the down kernel on one pair
+    (1, 8, 3, 256, 640, False),      # 15 of 16 waves used, 5 K slices per pair, 20 k tiles
+    (1, 8, 5, 128, 384, True),       # fp8 tiles of 64 k: 6 tiles over 3 waves per pair
+    (1, 16, 16, 128, 256, True),     # one wave per pair
+    (2, 3, 3, 128, 128, False),      # every token picks every expert
+    (5, 4, 2, 384, 128, True),       # K-sliced fp8 down projection with 4 k tiles per slice... (I/32 = 4)
+    (16, 2, 1, 128, 256, False),
+    (13, 64, 5, 256, 128, True),     # 65 routed pairs: one more than the in-kernel alignment takes
+])
+def test_fused_moe_odd_shapes(mlk, T, E, K, H, I, fp8):
+    _moe_case(mlk, T, E, K, H, I, torch.bfloat16, 1000 + T + K, fp8=fp8)
+
+
 def test_fused_moe_single_token_expert_map(mlk):
     """A routed expert that is not held locally contributes nothing."""
     from muxi_native_layout_kernels_amd.moe_planC import fused_moe
