@@ -1031,8 +1031,9 @@ __global__ void __launch_bounds__(256) moe_combine_kernel(const float *__restric
                                                           const int32_t *__restrict__ topk_ids,
                                                           const int32_t *__restrict__ experts_map, int K, int H,
                                                           int E, int SKD) {
+    // grid (tokens, chunks of 1024 outputs): one f32x4 cell per thread
     const int tok = blockIdx.x;
-    for (int n = threadIdx.x * 4; n < H; n += blockDim.x * 4) {
+    for (int n = (blockIdx.y * blockDim.x + threadIdx.x) * 4; n < H; n += gridDim.y * blockDim.x * 4) {
         f32x4 sum = {0.f, 0.f, 0.f, 0.f};
         for (int k = 0; k < K; ++k) {
             int e = topk_ids[tok * K + k];
@@ -1152,11 +1153,11 @@ static int launch_moe_tile(const MoeArgs &a, int max_tasks, float *obuf, hipStre
         while (skd < kMoeMaxKSlices && row_tiles * max_tasks * skd < 512 && windows % (skd * 2) == 0) skd *= 2;
         moe_down_tile_kernel<T, FP8, CB, R><<<dim3(row_tiles, max_tasks, skd), 256, tile_lds_bytes<CB>(), s>>>(a, obuf);
         MLK_LAUNCH_CHECK();
-        moe_combine_kernel<T><<<a.T, 256, 0, s>>>(obuf, a.Y, a.topk_ids, a.experts_map, a.K, a.H, a.E, skd);
+        moe_combine_kernel<T><<<dim3(a.T, (a.H + 1023) / 1024), 256, 0, s>>>(obuf, a.Y, a.topk_ids, a.experts_map, a.K, a.H, a.E, skd);
     } else {
         moe_down_tile_kernel<T, FP8, CB, 1><<<dim3(groups_h / kTileWaves, max_tasks, 1), 256, tile_lds_bytes<CB>(), s>>>(a, obuf);
         MLK_LAUNCH_CHECK();
-        moe_combine_kernel<T><<<a.T, 256, 0, s>>>(obuf, a.Y, a.topk_ids, a.experts_map, a.K, a.H, a.E, 1);
+        moe_combine_kernel<T><<<dim3(a.T, (a.H + 1023) / 1024), 256, 0, s>>>(obuf, a.Y, a.topk_ids, a.experts_map, a.K, a.H, a.E, 1);
     }
     MLK_LAUNCH_CHECK();
     return MLK_OK;
