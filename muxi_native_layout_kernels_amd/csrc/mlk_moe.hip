@@ -23,6 +23,8 @@
 // Algorithmic traffic per layer: active experts * 3*I*H*sizeof(W) (+ scales)
 // + 2*T*H*2 + T*E*2 bytes; the SiLU intermediate (T*K*I*2 bytes, written and
 // read once) stays in L2 / Infinity Cache for decode-sized T.
+#include <math.h>
+
 #include "mlk_tile.cuh"
 
 namespace mlk {
@@ -33,10 +35,16 @@ constexpr int kMoeChunk = 256;     // tokens per expert-compute pass
 static int g_moe_gemv1 = 1;        // experiment switch: GeMV-style kernels for a single token
 static int g_moe_tile = 1;         // experiment switch: row-shared kernels for tasks of more than one token block
 static inline bool moe_tile_path() { return g_moe_tile != 0; }
-// Token blocks per task: as many as the largest possible expert load needs, at most 8 with the
-// row-shared kernels (4 without); 5 and 7 round up to the next instantiated width.
-static inline int moe_blocks_per_task(int tokens) {
-    int cb = (tokens + 15) / 16;
+// Token blocks per task (the tokens of one expert that share a weight pass).  Sized for the load an
+// expert sees under even routing plus three standard deviations, not for the worst case: a hotter
+// expert simply gets a second task (a second pass over its weights), while every task of the launch
+// pays staging work for the full width.  At most 8 with the row-shared kernels (4 without); 5 and 7
+// round up to the next instantiated width.
+static inline int moe_blocks_per_task(int tokens, int topk, int experts) {
+    const double mean = (double)tokens * topk / experts;
+    int expect = (int)(mean + 3.0 * sqrt(mean)) + 1;
+    if (expect > tokens) expect = tokens;
+    int cb = (expect + 15) / 16;
     const int cap = moe_tile_path() ? 8 : 4;
     if (cb > cap) cb = cap;
     if (cb == 5) cb = 6;
@@ -1256,7 +1264,7 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
     for (int t0 = 0; t0 < n_tokens; t0 += kMoeChunk) {
         const int tc = n_tokens - t0 < kMoeChunk ? n_tokens - t0 : kMoeChunk;
         const int n_pairs = tc * topk;
-        const int cb = moe_blocks_per_task(tc);                  // an expert sees at most tc tokens
+        const int cb = moe_blocks_per_task(tc, topk, n_experts);
         MoeWorkspace ws;
         carve((uint8_t *)workspace, tc, n_experts, topk, hidden, inter, &ws);
         const int max_padded = n_pairs + n_experts * 15;
