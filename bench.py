@@ -204,6 +204,39 @@ def main():
                     active_experts=e_act, roofline_us=algo / HBM_PEAK_GBPS / 1e3,
                     ratio_to_roofline=us / (algo / HBM_PEAK_GBPS / 1e3), wall=wall)
 
+    def moe_next_case(name, T, steps, warmup):
+        """The routing configuration the reference's own router is written for (256 experts in 8 groups, 4 groups
+        kept, top-8, sigmoid scores with a selection bias) on expert matrices of H = 7168, I = 2048."""
+        E, K, H, I = 256, 8, 7168, 2048
+        if "next" not in moe_w:
+            moe_w.clear()
+            torch.cuda.empty_cache()
+            w1 = torch.empty((E, 2 * I, H), dtype=torch.bfloat16, device=dev)
+            w2 = torch.empty((E, H, I), dtype=torch.bfloat16, device=dev)
+            for e0 in range(0, E, 16):
+                w1[e0:e0 + 16] = (torch.randn((16, 2 * I, H), generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+                w2[e0:e0 + 16] = (torch.randn((16, H, I), generator=gen, device=dev) * 0.02).to(torch.bfloat16)
+            moe_w["next"] = (w1, w2, None, None)
+        w1, w2, _, _ = moe_w["next"]
+        x = torch.randn((T, H), generator=gen, device=dev).to(torch.bfloat16)
+        logits = torch.randn((T, E), generator=gen, device=dev).to(torch.bfloat16)
+        bias = (torch.randn((E,), generator=gen, device=dev) * 0.05).abs().to(torch.bfloat16)
+
+        def call():
+            return fused_moe(x, w1, w2, logits, K, True, use_grouped_topk=True, num_expert_group=8, topk_group=4,
+                             gating_bias=bias, score_func="sigmoid")
+        y = call()
+        ids = torch.empty((T, K), dtype=torch.int32, device=dev)
+        wts = torch.empty((T, K), dtype=torch.bfloat16, device=dev)
+        mlk.fused_routing_gate(logits, 1, T, H, 8, 4, ids, wts, K, bias)
+        e_act = int(torch.unique(ids).numel())
+        us, wall = run_graph([call], steps, warmup)
+        algo = e_act * 3 * I * H * 2 + 2 * T * H * 2 + T * E * 2
+        del y
+        return dict(name=name, us=us, bytes=algo, gbps=algo / us / 1e3, frac=algo / us / 1e3 / HBM_PEAK_GBPS,
+                    active_experts=e_act, roofline_us=algo / HBM_PEAK_GBPS / 1e3,
+                    ratio_to_roofline=us / (algo / HBM_PEAK_GBPS / 1e3), wall=wall)
+
     if args.calibrate_copy:
         src = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -249,6 +282,8 @@ def main():
             per_config.append(moe_case("C5 bf16 fused_moe T=%d" % T, T, False, 20, 5))
         for T in (1, 16):
             per_config.append(moe_case("C5 soft-fp8 fused_moe T=%d" % T, T, True, 20, 5))
+        for T in (1, 16):
+            per_config.append(moe_next_case("next: grouped-routing MoE E=256 top-8 H=7168 I=2048 bf16 T=%d" % T, T, 20, 5))
         moe_w.clear()
         torch.cuda.empty_cache()
         for row in per_config:

@@ -234,6 +234,16 @@ def test_fused_moe_odd_shapes(mlk, T, E, K, H, I, fp8):
     _moe_case(mlk, T, E, K, H, I, torch.bfloat16, 1000 + T + K, fp8=fp8)
 
 
+@pytest.mark.parametrize("T", [1, 4, 16, 40])
+@pytest.mark.parametrize("fp8", [False, True])
+def test_fused_moe_deepseek_style_routing(mlk, T, fp8):
+    """256 experts in 8 groups, 4 groups kept, top-8, sigmoid scores with a selection bias - the only routing
+    configuration the reference's own router accepts (fused_gating.h:22-34, test_muxi_moe.py:41-50)."""
+    E = 256
+    bias = randn((E,), torch.bfloat16, 0.05, 77).abs()
+    _moe_case(mlk, T, E, 8, 256, 128, torch.bfloat16, 1200 + T, score="sigmoid", groups=(8, 4), bias=bias, fp8=fp8)
+
+
 def test_fused_moe_single_token_expert_map(mlk):
     """A routed expert that is not held locally contributes nothing."""
     from muxi_native_layout_kernels_amd.moe_planC import fused_moe
