@@ -117,7 +117,7 @@ int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k
                       int p2, void *stream);
 
 /* --------------------------------------------------------------- narrow GeMM
- * C = T(alpha * B . A^T (+ bias[N])), 1 <= M <= 256, A in layout-A, MFMA
+ * C = T(alpha * B . A^T (+ bias[N])), any M >= 1 (in passes over the weights), A in layout-A, MFMA
  * 16x16x32 with fp32 accumulation.
  *
  *   b_mode MLK_B_ROWMAJOR, c_mode MLK_C_ROWMAJOR : `gemm_layoutA` / `_wapper`
@@ -137,7 +137,8 @@ int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k
  *   kernel_id 2  row-shared kernel: four waves walk the same k tiles and share the activations
  *                of each k window through LDS (p2 is ignored); falls back to kernel 1 for a
  *                shape it does not tile (N/16 not a multiple of 4 p1, or K/32 not a multiple
- *                of 4 p3)
+ *                of 4 p3).  With row-major B and C it takes more than 64 tokens in passes of up
+ *                to 128 (p1 limited to 2) instead of 64
  *   kernel_id 12, 14, 16, 18  kernel 1 with 2, 4, 6 or 8 k tiles in flight per wave instead of the
  *                default depth; honoured for up to 16 tokens with row-major B and C, otherwise
  *                the same as kernel 1

@@ -111,6 +111,9 @@ def _gemv_default(n, k):
 def _gemm_default(n, m, k):
     """Fallback for a GEMM shape that was never scanned."""
     groups = max(1, n // 16)
+    if m > 64 and groups % 4 == 0 and (k // 32) % 2 == 0:
+        # more than 64 tokens: the row-shared kernel takes 128 tokens per pass over the weights
+        return (2, 2 if groups % 8 == 0 else 1, 1, 2 if (k // 32) % 4 == 0 else 1)
     r = 1 if m > 32 else 2
     if groups % r:
         r = 1

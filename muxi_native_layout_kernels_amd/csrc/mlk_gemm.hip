@@ -28,7 +28,7 @@ extern "C" size_t mlk_gemm_counter_bytes(void) { return kCounterBytes; }
 extern "C" size_t mlk_gemm_workspace_bytes(int m, int n, int p1, int p3) {
     (void)p1;
     int cb = (m + 15) / 16;
-    if (cb > 4) cb = 4;
+    if (cb > 8) cb = 8;                                  // kernel 2 takes up to 128 tokens per weight pass
     if (p3 <= 1) return 0;
     return kCounterBytes + (size_t)p3 * (size_t)(n / 16) * cb * 1024;
 }
@@ -64,7 +64,7 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
     MLK_REQUIRE(a && b && c, "gemm: null pointer");
     int sk = p3;
     if (sk > k / 32) sk = k / 32 > 0 ? k / 32 : 1;
-    const int cb_max = (m + 15) / 16 < 4 ? (m + 15) / 16 : 4;
+    const int cb_max = (m + 15) / 16 < 8 ? (m + 15) / 16 : 8;
     if (sk > 1) {
         MLK_REQUIRE(workspace != nullptr, "gemm: a K split across workgroups needs a workspace");
         MLK_REQUIRE((size_t)(n / 16 / p1) * sizeof(int) <= kCounterBytes, "gemm: too many row tiles for the counter region");
@@ -91,9 +91,14 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
     g.rotate = g_tunable[0];
     g.depth = kernel_id >= 12 ? kernel_id - 10 : 0;
     hipStream_t s = (hipStream_t)stream;
-    // weight passes of at most 64 tokens
-    for (int c0 = 0; c0 < m; c0 += 64) {
-        int mm = m - c0 < 64 ? m - c0 : 64;
+    // weight passes of at most 64 tokens; 128 with the row-shared kernel on row-major operands when it tiles
+    // the shape with two k tiles per window
+    int pass = 64;
+    if (kernel_id == 2 && m > 64 && b_mode == MLK_B_ROWMAJOR && c_mode == MLK_C_ROWMAJOR &&
+        (n / 16) % (kTileWaves * (p1 >= 2 ? 2 : 1)) == 0 && (k / 32) % (sk * 2) == 0)
+        pass = 128;
+    for (int c0 = 0; c0 < m; c0 += pass) {
+        int mm = m - c0 < pass ? m - c0 : pass;
         g.M = mm;
         g.cb0 = c0 / 16;
         int cb = (mm + 15) / 16;

@@ -366,11 +366,13 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(GemmArgs p) {
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    TileLoop<T, FP8, CB, R>::run(acc, abase, srow, bs, tbeg, tend, tile_win, p.rotate ? rt : 0);
+    const int nb = (p.M + 15) >> 4;                       // token blocks of this launch (<= CB)
+    TileLoop<T, FP8, CB, R>::run(acc, abase, srow, bs, tbeg, tend, tile_win, p.rotate ? rt : 0, nb);
 
     constexpr int NTILE = R * CB;
     const int row_tiles = gridDim.x / p.SK;
     auto epilogue = [&](int r, int cb, f32x4 v) {
+        if (cb >= nb) return;
         const int n = (rg0 + r) * 16 + 4 * q;
         const int tok = (p.cb0 + cb) * 16 + r16;
         if (tok >= p.M_total) return;
@@ -422,9 +424,10 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(GemmArgs p) {
 }
 
 // Can kernel 2 run this problem with these parameters?
-static bool tile_kernel_fits(const GemmArgs &p, int R) {
+static bool tile_kernel_fits(const GemmArgs &p, int R, int CB) {
     const int tiles_total = p.K / 32;
-    return (p.N / 16) % (kTileWaves * R) == 0 && p.SK >= 1 && tiles_total % (p.SK * kTileKW) == 0;  // CB <= 4 here
+    const int kw = CB > 4 ? 2 : 4;                       // tile_kw<CB>()
+    return (p.N / 16) % (kTileWaves * R) == 0 && p.SK >= 1 && tiles_total % (p.SK * kw) == 0;
 }
 
 template <class T, bool FP8, int CB, int R, int BMODE, int CMODE>
@@ -477,12 +480,21 @@ template <class T, bool FP8, int BMODE, int CMODE>
 static int launch_rc(const GemmArgs &p, int kernel_id, int R, int CB, hipStream_t s) {
 #define MLK_CASE(RR, CC)                                                                        \
     if (R == RR && CB == CC)                                                                    \
-        return (kernel_id == 2 && tile_kernel_fits(p, RR)) ? launch_tile<T, FP8, CC, RR, BMODE, CMODE>(p, s) \
+        return (kernel_id == 2 && tile_kernel_fits(p, RR, CC)) ? launch_tile<T, FP8, CC, RR, BMODE, CMODE>(p, s) \
                                                           : launch<T, FP8, CC, RR, BMODE, CMODE>(p, s);
     MLK_CASE(1, 1) MLK_CASE(1, 2) MLK_CASE(1, 3) MLK_CASE(1, 4)
     MLK_CASE(2, 1) MLK_CASE(2, 2) MLK_CASE(2, 3) MLK_CASE(2, 4)
     MLK_CASE(4, 1) MLK_CASE(4, 2) MLK_CASE(4, 3) MLK_CASE(4, 4)
 #undef MLK_CASE
+    // five to eight token blocks (up to 128 tokens per weight pass): row-shared kernel, row-major B and C
+    if constexpr (BMODE == MLK_B_ROWMAJOR && CMODE == MLK_C_ROWMAJOR) {
+        if (CB > 4) {
+            const int rr = R >= 2 ? 2 : 1;
+            if (!tile_kernel_fits(p, rr, CB)) return fail(MLK_ERR_INVALID, "gemm: wide pass does not tile this shape");
+            if (CB <= 6) return rr == 2 ? launch_tile<T, FP8, 6, 2, BMODE, CMODE>(p, s) : launch_tile<T, FP8, 6, 1, BMODE, CMODE>(p, s);
+            return rr == 2 ? launch_tile<T, FP8, 8, 2, BMODE, CMODE>(p, s) : launch_tile<T, FP8, 8, 1, BMODE, CMODE>(p, s);
+        }
+    }
     // eight row groups per wave: wave kernel only; more than one token block only with row-major B and C
     if (R == 8 && CB == 1) return launch<T, FP8, 1, 8, BMODE, CMODE>(p, s);
     if constexpr (BMODE == MLK_B_ROWMAJOR && CMODE == MLK_C_ROWMAJOR) {

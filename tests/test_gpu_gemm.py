@@ -114,6 +114,38 @@ def test_gemm_ring_depth_soft_fp8(mlk):
             assert_close(c, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), b), RTOL, ATOL, "fp8 depth")
 
 
+@pytest.mark.parametrize("m", [65, 100, 128, 130, 200, 256, 300])
+@pytest.mark.parametrize("p1,p3", [(1, 1), (2, 1), (2, 2), (4, 4)])
+def test_gemm_tile_kernel_wide_passes(mlk, m, p1, p3):
+    """More than 64 tokens with kernelId 2 on row-major operands: passes of up to 128 tokens over the weights."""
+    n, k = 512, 1024
+    w = randn((n, k), torch.bfloat16, 0.02, 51)
+    b = randn((m, k), torch.bfloat16, 1.0, 52)
+    bias = randn((1, n), torch.bfloat16, 1.0, 53)
+    a = pack_a(w).cuda()
+    c = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=p1, kernelParam2=1, kernelParam3=p3,
+                                kernelId=2, bias=bias.cuda())
+    assert_close(c, ogemm.linear_expected(w, b, 0.5, bias), RTOL, ATOL, "wide passes M=%d" % m)
+    c2 = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=p1, kernelParam2=1, kernelParam3=p3,
+                                 kernelId=2, bias=bias.cuda())
+    assert torch.equal(c, c2)
+
+
+def test_gemm_wide_default_parameters(mlk):
+    """A shape that is in no table: above 64 tokens the heuristic picks the row-shared kernel."""
+    n, k, m = 768, 512, 150
+    w = randn((n, k), torch.float16, 0.02, 61)
+    b = randn((m, k), torch.float16, 1.0, 62)
+    c = mlk.gemm_layoutA(pack_a(w).cuda(), b.cuda())
+    assert_close(c, ogemm.linear_expected(w, b), RTOL, ATOL, "wide default")
+    codes = fp8_codes((n, k), 63)
+    g = torch.Generator().manual_seed(64)
+    scale = (torch.rand((n // 128, k // 128), generator=g) * 0.02 + 0.001).float()
+    bb = randn((m, k), torch.bfloat16, 1.0, 65)
+    c8 = mlk.gemm_layoutA_linear(pack_a(codes).cuda(), bb.cuda(), scale_matrix=scale.cuda())
+    assert_close(c8, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), bb), RTOL, ATOL, "wide default fp8")
+
+
 def test_gemm_special_cases(mlk):
     n = k = 256
     eye = torch.eye(n, dtype=torch.float16)
