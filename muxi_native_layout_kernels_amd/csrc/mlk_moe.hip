@@ -53,19 +53,56 @@ static inline int moe_blocks_per_task(int tokens, int topk, int experts) {
 }
 
 // ------------------------------------------------------------------ router
+// Largest value of the wave, in every lane: four rotations inside the rows of 16 lanes on the DPP
+// path, then the four row results through scalar registers.
+__device__ __forceinline__ uint32_t wave_max_u32(uint32_t v) {
+    v = max(v, (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x128, 0xf, 0xf, true));   // row_ror:8
+    v = max(v, (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x124, 0xf, 0xf, true));   // row_ror:4
+    v = max(v, (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x122, 0xf, 0xf, true));   // row_ror:2
+    v = max(v, (uint32_t)__builtin_amdgcn_mov_dpp((int)v, 0x121, 0xf, 0xf, true));   // row_ror:1
+    const uint32_t a = __builtin_amdgcn_readlane((int)v, 0), b = __builtin_amdgcn_readlane((int)v, 16);
+    const uint32_t c = __builtin_amdgcn_readlane((int)v, 32), d = __builtin_amdgcn_readlane((int)v, 48);
+    return max(max(a, b), max(c, d));
+}
+
+// unsigned keys in the order of the floats (-0 counts as +0), and back
+__device__ __forceinline__ uint32_t order_key(float f) {
+    uint32_t b = __float_as_uint(f);
+    if ((b << 1) == 0u) b = 0u;
+    return (b & 0x80000000u) ? ~b : (b | 0x80000000u);
+}
+__device__ __forceinline__ float order_key_value(uint32_t k) {
+    return __uint_as_float((k & 0x80000000u) ? (k ^ 0x80000000u) : ~k);
+}
+
+// One round of "take the largest, ties to the lower index": the values sit in registers (index
+// lane + 64 i).  Two wave reductions on the DPP path - no LDS, no barrier.  Returns the index.
+template <int NE>
+__device__ __forceinline__ uint32_t wave_argmax(const float (&v)[NE], int lane) {
+    uint32_t bk = order_key(v[0]);
+    uint32_t bi = (uint32_t)lane;
+#pragma unroll
+    for (int i = 1; i < NE; ++i) {
+        const uint32_t k = order_key(v[i]);
+        if (k > bk) { bk = k; bi = (uint32_t)(lane + 64 * i); }
+    }
+    const uint32_t top = wave_max_u32(bk);
+    return ~wave_max_u32(~(bk == top ? bi : 0xffffffffu));   // lowest index among the holders
+}
+
+// One wave per token.  Expert lane + 64 i lives in register slot i of its lane.
 template <class T>
 __global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__ logits, int n_tokens, int E,
                                                     int n_groups, int topk_groups, int topk, int score_fun,
                                                     const uint16_t *__restrict__ bias, int renorm,
                                                     int32_t *__restrict__ ids, uint16_t *__restrict__ weights) {
-    __shared__ double ex[kMaxExperts];     // logits, then exp(x - max)
-    __shared__ float prob[kMaxExperts];    // un-biased score rounded to T
-    __shared__ float sel[kMaxExperts];     // selection score rounded to T
-    __shared__ float gscore[kMaxExperts];
+    __shared__ __align__(16) double ex[kMaxExperts];   // exp(x - max), for the index-order sum
+    __shared__ __align__(16) float sel[kMaxExperts];   // selection scores, for the group scores
     __shared__ int keep[kMaxExperts];
-    __shared__ double s_sum;
     __shared__ int pick_id[kMaxTopK];
     __shared__ float pick_w[kMaxTopK];
+    constexpr int NE = kMaxExperts / 64;
+    constexpr float kLowest = -3.0e38f;
 
     const int tok = blockIdx.x;
     const int lane = threadIdx.x;
@@ -73,117 +110,146 @@ __global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__
     auto round_T = [](float v) { return T::to_f32(T::from_f32(v)); };
 
     // scores: exp, the index-order sum and the division in float64, one rounding to fp32, one to T
-    double mx = -1.0e300;
-    for (int j = lane; j < E; j += 64) {
-        double v = (double)T::to_f32(row[j]);
-        ex[j] = v;
-        mx = fmax(mx, v);
+    float xv[NE];
+    float lmax = kLowest;
+#pragma unroll
+    for (int i = 0; i < NE; ++i) {
+        const int j = lane + 64 * i;
+        xv[i] = j < E ? T::to_f32(row[j]) : kLowest;
+        lmax = fmaxf(lmax, xv[i]);
     }
-    for (int m = 32; m >= 1; m >>= 1) {
-        double o = __shfl_xor(mx, m);
-        mx = fmax(mx, o);
-    }
+    float pv[NE], sv[NE];      // un-biased score and selection score, both rounded to T
     if (score_fun == 0) {
-        for (int j = lane; j < E; j += 64) ex[j] = exp(ex[j] - mx);
+        const double mx = (double)order_key_value(wave_max_u32(order_key(lmax)));
+        double ev[NE];
+#pragma unroll
+        for (int i = 0; i < NE; ++i) ev[i] = lane + 64 * i < E ? exp((double)xv[i] - mx) : 0.0;
+        // The sum runs over the experts in index order, the same in every lane: the terms go through
+        // LDS and come back sixteen at a time (eight 16-byte reads in flight), then add in order.
+#pragma unroll
+        for (int i = 0; i < NE; ++i)
+            if (lane + 64 * i < E) ex[lane + 64 * i] = ev[i];
         __syncthreads();
-        if (lane == 0) {
-            double s = 0.0;
-            for (int j = 0; j < E; ++j) s += ex[j];
-            s_sum = s;
-        }
-        __syncthreads();
-        const double s = s_sum;
-        for (int j = lane; j < E; j += 64) prob[j] = round_T((float)(ex[j] / s));
-    } else {
-        for (int j = lane; j < E; j += 64) prob[j] = round_T((float)(1.0 / (1.0 + exp(-ex[j]))));
-    }
-    for (int j = lane; j < E; j += 64) sel[j] = bias ? round_T(prob[j] + T::to_f32(bias[j])) : prob[j];
-    __syncthreads();
-
-    // group scores: max of the group, or the T-sum of its two largest positive scores with a bias
-    const int per_group = E / n_groups;
-    for (int g = lane; g < n_groups; g += 64) {
-        const float *seg = sel + g * per_group;
-        float score;
-        if (!bias) {
-            score = 0.f;
-            for (int j = 0; j < per_group; ++j) score = seg[j] > score ? seg[j] : score;
-        } else {
-            float a = 0.f, b = 0.f;  // largest, second largest positive
-            for (int j = 0; j < per_group; ++j) {
-                float v = seg[j];
-                if (v > a) { b = a; a = v; }
-                else if (v > b) b = v;
+        typedef __attribute__((ext_vector_type(2))) double f64x2;
+        double s = 0.0;
+        for (int j0 = 0; j0 < E; j0 += 16) {
+            f64x2 r[8];
+#pragma unroll
+            for (int t = 0; t < 8; ++t) r[t] = *reinterpret_cast<const f64x2 *>(&ex[j0 + 2 * t]);
+#pragma unroll
+            for (int t = 0; t < 8; ++t) {
+                if (j0 + 2 * t < E) s += r[t][0];
+                if (j0 + 2 * t + 1 < E) s += r[t][1];
             }
-            score = 0.f;
-            if (a > 0.f) score = round_T(a + score);
-            if (b > 0.f) score = round_T(b + score);
         }
-        gscore[g] = score;
-        keep[g] = 0;
+#pragma unroll
+        for (int i = 0; i < NE; ++i) pv[i] = round_T((float)(ev[i] / s));
+    } else {
+#pragma unroll
+        for (int i = 0; i < NE; ++i) pv[i] = round_T((float)(1.0 / (1.0 + exp(-(double)xv[i]))));
     }
-    __syncthreads();
-    if (lane == 0) {
-        for (int i = 0; i < topk_groups; ++i) {
-            int best = 0;
-            for (int g = 1; g < n_groups; ++g)
-                if (gscore[g] > gscore[best]) best = g;
-            keep[best] = 1;
-            gscore[best] = 0.f;
+#pragma unroll
+    for (int i = 0; i < NE; ++i) {
+        const int j = lane + 64 * i;
+        sv[i] = (bias && j < E) ? round_T(pv[i] + T::to_f32(bias[j])) : pv[i];
+        if (j >= E) { sv[i] = kLowest; pv[i] = 0.f; }
+    }
+
+    if (n_groups > 1) {
+        // group scores: max of the group, or the T-sum of its two largest positive scores with a bias
+#pragma unroll
+        for (int i = 0; i < NE; ++i)
+            if (lane + 64 * i < E) sel[lane + 64 * i] = sv[i];
+        __syncthreads();
+        const int per_group = E / n_groups;
+        float gs[NE];
+        int kept[NE];
+#pragma unroll
+        for (int i = 0; i < NE; ++i) {
+            const int g = lane + 64 * i;
+            gs[i] = kLowest;
+            kept[i] = 0;
+            if (g < n_groups) {
+                const float *seg = sel + g * per_group;
+                float score = 0.f;
+                if (!bias) {
+#pragma unroll 8
+                    for (int j = 0; j < per_group; ++j) score = seg[j] > score ? seg[j] : score;
+                } else {
+                    float a = 0.f, b = 0.f;  // largest, second largest positive
+#pragma unroll 8
+                    for (int j = 0; j < per_group; ++j) {
+                        float v = seg[j];
+                        if (v > a) { b = a; a = v; }
+                        else if (v > b) b = v;
+                    }
+                    if (a > 0.f) score = round_T(a + score);
+                    if (b > 0.f) score = round_T(b + score);
+                }
+                gs[i] = score;
+            }
+        }
+        // keep the topk_groups best groups: largest score, ties to the lower group, a kept score becomes 0
+        for (int t = 0; t < topk_groups; ++t) {
+            const uint32_t pick = wave_argmax<NE>(gs, lane);
+            if ((int)(pick & 63u) == lane) {
+#pragma unroll
+                for (int i = 0; i < NE; ++i)
+                    if (i == (int)(pick >> 6)) { gs[i] = 0.f; kept[i] = 1; }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < NE; ++i)
+            if (lane + 64 * i < n_groups) keep[lane + 64 * i] = kept[i];
+        __syncthreads();
+#pragma unroll
+        for (int i = 0; i < NE; ++i) {
+            const int j = lane + 64 * i;
+            if (j < E && !keep[j / per_group]) { sv[i] = 0.f; pv[i] = 0.f; }
         }
     }
-    __syncthreads();
-    for (int j = lane; j < E; j += 64)
-        if (!keep[j / per_group]) { sel[j] = 0.f; prob[j] = 0.f; }
-    __syncthreads();
 
     // K rounds of arg-max over the selection scores, ties to the lower id; a picked score becomes 0
     for (int kk = 0; kk < topk; ++kk) {
-        float bv = sel[lane < E ? lane : 0];
-        int bi = lane < E ? lane : 0;
-        for (int j = lane + 64; j < E; j += 64)
-            if (sel[j] > bv) { bv = sel[j]; bi = j; }
-        if (lane >= E) { bv = -3.0e38f; bi = 0x7fffffff; }
-        for (int m = 32; m >= 1; m >>= 1) {
-            float ov = __shfl_xor(bv, m);
-            int oi = __shfl_xor(bi, m);
-            if (ov > bv || (ov == bv && oi < bi)) { bv = ov; bi = oi; }
+        const uint32_t pick = wave_argmax<NE>(sv, lane);
+        if ((int)(pick & 63u) == lane) {
+            pick_id[kk] = (int)pick;
+#pragma unroll
+            for (int i = 0; i < NE; ++i)
+                if (i == (int)(pick >> 6)) { pick_w[kk] = pv[i]; sv[i] = 0.f; }
         }
-        if (lane == 0) {
-            pick_id[kk] = bi;
-            pick_w[kk] = prob[bi];
-            sel[bi] = 0.f;
+    }
+    __syncthreads();
+
+    // Lane a now takes pick a.  The softmax variant returns its picks ordered by expert id (stable for
+    // equal ids): each lane counts the picks that go before its own and moves its pick there.
+    int my_id = lane < topk ? pick_id[lane] : 0x7fffffff;
+    float my_w = lane < topk ? pick_w[lane] : 0.f;
+    if (score_fun == 0) {
+        int before = 0;
+        for (int b = 0; b < topk; ++b) {
+            const int ib = __builtin_amdgcn_readlane(my_id, b);
+            before += (ib < my_id || (ib == my_id && b < lane)) ? 1 : 0;
         }
         __syncthreads();
+        if (lane < topk) {
+            pick_id[before] = my_id;
+            pick_w[before] = my_w;
+        }
+        __syncthreads();
+        my_id = lane < topk ? pick_id[lane] : 0x7fffffff;
+        my_w = lane < topk ? pick_w[lane] : 0.f;
     }
-
-    if (lane == 0) {
-        if (score_fun == 0) {
-            // the softmax variant returns its picks ordered by expert id
-            for (int a = 1; a < topk; ++a) {
-                int id = pick_id[a];
-                float w = pick_w[a];
-                int b = a - 1;
-                while (b >= 0 && pick_id[b] > id) {
-                    pick_id[b + 1] = pick_id[b];
-                    pick_w[b + 1] = pick_w[b];
-                    --b;
-                }
-                pick_id[b + 1] = id;
-                pick_w[b + 1] = w;
-            }
-        }
-        float denom = 1.f;
-        if (renorm) {
-            float s = 0.f;
-            for (int a = 0; a < topk; ++a) s += pick_w[a];
-            denom = round_T(s);
-        }
-        for (int a = 0; a < topk; ++a) {
-            ids[(size_t)tok * topk + a] = pick_id[a];
-            float w = renorm ? pick_w[a] / denom : pick_w[a];
-            weights[(size_t)tok * topk + a] = (uint16_t)T::from_f32(w);
-        }
+    float denom = 1.f;
+    if (renorm) {
+        float s = 0.f;      // fp32 sum in output order, the same in every lane
+        for (int a = 0; a < topk; ++a) s += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_w), a));
+        denom = round_T(s);
+    }
+    if (lane < topk) {
+        ids[(size_t)tok * topk + lane] = my_id;
+        const float w = renorm ? my_w / denom : my_w;
+        weights[(size_t)tok * topk + lane] = (uint16_t)T::from_f32(w);
     }
 }
 
