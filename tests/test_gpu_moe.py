@@ -49,6 +49,25 @@ def test_router_grouped_deepseek_configuration(mlk, dtype, score_fun, with_bias)
     assert torch.equal(w.view(torch.int16), w_o.view(torch.int16))
 
 
+@pytest.mark.parametrize("E,n_groups,topk_groups,K,score_fun,signed_bias", [
+    (256, 128, 70, 8, 1, False),     # more than 64 groups: a lane holds several groups
+    (256, 256, 40, 32, 0, False),    # one expert per group, the largest top-k
+    (96, 3, 2, 7, 0, True),          # E not a power of two, bias of both signs (negative selection scores)
+    (12, 4, 1, 3, 1, True),          # fewer candidates than picks inside the kept group: zeros are re-picked
+    (200, 8, 8, 10, 0, False),
+])
+def test_router_general_groupings(mlk, E, n_groups, topk_groups, K, score_fun, signed_bias):
+    T = 37
+    logits = randn((T, E), torch.bfloat16, 2.0, 900 + E)
+    bias = randn((E,), torch.bfloat16, 0.3, 901 + E) if signed_bias else None
+    for renorm in (False, True):
+        ids, w = _route_gpu(mlk, logits, score_fun, n_groups, topk_groups, K, bias, renorm=renorm)
+        ids_o, w_o = orouter.route(logits, score_fun, n_groups, topk_groups, K, bias)
+        assert torch.equal(ids, ids_o)
+        w_o = orouter.renormalize(w_o) if renorm else w_o
+        assert torch.equal(w.view(torch.int16), w_o.view(torch.int16))
+
+
 def test_router_special_cases_and_renorm(mlk):
     eq = torch.zeros((3, 16), dtype=torch.bfloat16)
     ids, w = _route_gpu(mlk, eq, 0, 1, 1, 4)
