@@ -366,7 +366,8 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(GemmArgs p) {
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) acc[r][cb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    const int nb = (p.M + 15) >> 4;                       // token blocks of this launch (<= CB)
+    // token blocks of this launch: exactly CB, except that 5 and 7 blocks run in the 6- and 8-wide instantiations
+    const int nb = CB > 4 ? (p.M + 15) >> 4 : CB;
     TileLoop<T, FP8, CB, R>::run(acc, abase, srow, bs, tbeg, tend, tile_win, p.rotate ? rt : 0, nb);
 
     constexpr int NTILE = R * CB;

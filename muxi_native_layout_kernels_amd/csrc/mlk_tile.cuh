@@ -134,14 +134,18 @@ struct TileLoop {
             if (do_stage) stage_load();
 #pragma unroll
             for (int w = 0; w < KW; ++w) {
-                u32x4 a[R];
+                // all fragment reads of the k tile go out first, then the products (the tests on nb
+                // are uniform: scalar branches)
+                u32x4 a[R], b[CB];
+#pragma unroll
+                for (int cb = 0; cb < CB; ++cb)
+                    if (cb < nb) b[cb] = win[slot * WG + (w * CB + cb) * 68 + q * 17 + r16];
                 weight_operands<FP8, R>(a, wf[slot][w], sc[slot][w]);
 #pragma unroll
                 for (int cb = 0; cb < CB; ++cb) {
-                    if (cb < nb) {                       // uniform: a scalar branch
-                        const u32x4 b = win[slot * WG + (w * CB + cb) * 68 + q * 17 + r16];
+                    if (cb < nb) {
 #pragma unroll
-                        for (int r = 0; r < R; ++r) acc[r][cb] = T::mfma(a[r], b, acc[r][cb]);
+                        for (int r = 0; r < R; ++r) acc[r][cb] = T::mfma(a[r], b[cb], acc[r][cb]);
                     }
                 }
             }
