@@ -48,8 +48,14 @@ struct GemmArgs {
     float alpha;
 };
 
+// Threads per workgroup the wave kernel is compiled for: deep register rings (many tiles x many
+// k tiles in flight) get the register budget of a 256-thread workgroup instead of spilling.
+__host__ __device__ constexpr int wave_kernel_threads(int ntile, int depth, bool staged) {
+    return (!staged && ntile * depth >= 24 && max_threads_for_tiles(ntile) > 256) ? 256 : max_threads_for_tiles(ntile);
+}
+
 template <class T, bool FP8, int CB, int R, int BMODE, int CMODE, int U, bool STAGE>
-__global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) gemm_wave_kernel(GemmArgs p) {
+__global__ void __launch_bounds__(wave_kernel_threads(R *CB, U, STAGE)) gemm_wave_kernel(GemmArgs p) {
     extern __shared__ f32x4 red[];  // [WK][R*CB][64]; the staged variant first uses it for two activation windows
     __shared__ int s_last;
 
@@ -447,7 +453,7 @@ static int launch(const GemmArgs &p, hipStream_t s) {
     int row_tiles = (q.N / 16) / R;
     int grid = row_tiles * q.SK;
     size_t lds = q.WK > 1 ? (size_t)q.WK * R * CB * 1024 : 0;
-    if constexpr (BMODE == MLK_B_ROWMAJOR) {
+    if constexpr (BMODE == MLK_B_ROWMAJOR && CB >= 3) {
         // stage row-major activations through LDS when every K slice is a whole number of WK-tile windows
         const int tiles_total = q.K / 32;
         const int tiles_per = (tiles_total + q.SK - 1) / q.SK;
@@ -465,6 +471,7 @@ static int launch(const GemmArgs &p, hipStream_t s) {
         // kernel ids 12, 14, 16, 18: explicit depth of the register ring (k tiles in flight per wave)
 #define MLK_DEPTH(UU)                                                                                   \
     if (q.depth == UU) {                                                                                \
+        while (q.WK * 64 > wave_kernel_threads(R * CB, UU, false)) q.WK >>= 1;                          \
         gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, UU, false><<<grid, q.WK * 64, lds, s>>>(q);       \
         MLK_LAUNCH_CHECK();                                                                             \
         return MLK_OK;                                                                                  \
