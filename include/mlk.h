@@ -139,6 +139,12 @@ int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k
  *                shape it does not tile (N/16 not a multiple of 4 p1, or K/32 not a multiple
  *                of 4 p3).  With row-major B and C it takes more than 64 tokens in passes of up
  *                to 128 (p1 limited to 2) instead of 64
+ *   kernel_id 4  kernel 1 with one workgroup per CU: the N/16 row groups are dealt out as evenly as
+ *                possible, two to four per workgroup (p1 and p3 are ignored).  What one CU can pull
+ *                through its memory path bounds these kernels, so for few weight rows an even
+ *                deal over all CUs beats a fixed p1.  16-bit weights, row-major B and C, up to 32
+ *                tokens per pass, N/16 above the CU count and at most four times it; otherwise
+ *                the same as kernel 1
  *   kernel_id 12, 14, 16, 18  kernel 1 with 2, 4, 6 or 8 k tiles in flight per wave instead of the
  *                default depth; honoured for up to 16 tokens with row-major B and C, otherwise
  *                the same as kernel 1

@@ -40,7 +40,7 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
     MLK_REQUIRE(m >= 0 && n >= 0 && k >= 0, "gemm: negative size");
     MLK_REQUIRE(n % 16 == 0, "gemm: N % 16 must be 0");
     MLK_REQUIRE(k % 32 == 0, "gemm: K % 32 must be 0");
-    MLK_REQUIRE(kernel_id == 1 || kernel_id == 2 || kernel_id == 12 || kernel_id == 14 || kernel_id == 16 ||
+    MLK_REQUIRE(kernel_id == 1 || kernel_id == 2 || kernel_id == 4 || kernel_id == 12 || kernel_id == 14 || kernel_id == 16 ||
                     kernel_id == 18,
                 "gemm: unknown kernel id");
     MLK_REQUIRE(p1 == 1 || p1 == 2 || p1 == 4 || p1 == 8, "gemm: row groups per wave (p1) must be 1, 2, 4 or 8");

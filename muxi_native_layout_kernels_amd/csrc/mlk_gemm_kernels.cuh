@@ -54,17 +54,14 @@ __host__ __device__ constexpr int wave_kernel_threads(int ntile, int depth, bool
     return (!staged && ntile * depth >= 24 && max_threads_for_tiles(ntile) > 256) ? 256 : max_threads_for_tiles(ntile);
 }
 
+// The body of the wave kernel for the R row groups from rg0 (row tile rt of `row_tiles`, K slice sk).
+// red: [WK][R*CB][64] f32x4 of LDS; the staged variant first uses it for two activation windows.
 template <class T, bool FP8, int CB, int R, int BMODE, int CMODE, int U, bool STAGE>
-__global__ void __launch_bounds__(wave_kernel_threads(R *CB, U, STAGE)) gemm_wave_kernel(GemmArgs p) {
-    extern __shared__ f32x4 red[];  // [WK][R*CB][64]; the staged variant first uses it for two activation windows
-    __shared__ int s_last;
-
+__device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, const int sk, const int rg0,
+                                               const int row_tiles, f32x4 *red, int &s_last) {
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);  // wave-uniform, kept scalar
     const int q = lane >> 4, r16 = lane & 15;
-    const int sk = blockIdx.x % p.SK;
-    const int rt = blockIdx.x / p.SK;
-    const int rg0 = rt * R;
     const int tiles_total = p.K >> 5;
     const int tiles_per = (tiles_total + p.SK - 1) / p.SK;
     const int tbeg = sk * tiles_per;
@@ -250,7 +247,6 @@ __global__ void __launch_bounds__(wave_kernel_threads(R *CB, U, STAGE)) gemm_wav
     mfma_settle();
 
     constexpr int NTILE = R * CB;
-    const int row_tiles = gridDim.x / p.SK;
 
     auto epilogue = [&](int j, f32x4 v) {
         const int r = j / CB, cb = j - r * CB;
@@ -321,6 +317,31 @@ __global__ void __launch_bounds__(wave_kernel_threads(R *CB, U, STAGE)) gemm_wav
         for (int s = 0; s < p.SK; ++s) v += ld_agent_f32x4(&part[part_at(s, j)]);
         epilogue(j, v);
     }
+}
+
+template <class T, bool FP8, int CB, int R, int BMODE, int CMODE, int U, bool STAGE>
+__global__ void __launch_bounds__(wave_kernel_threads(R *CB, U, STAGE)) gemm_wave_kernel(GemmArgs p) {
+    extern __shared__ f32x4 red[];
+    __shared__ int s_last;
+    const int rt = blockIdx.x / p.SK;
+    gemm_wave_body<T, FP8, CB, R, BMODE, CMODE, U, STAGE>(p, rt, blockIdx.x % p.SK, rt * R, gridDim.x / p.SK, red, s_last);
+}
+
+// Kernel id 4: one workgroup per CU, the row groups dealt out as evenly as possible, so a workgroup
+// owns floor or ceil(groups / grid) consecutive row groups: RMAX or RMAX - 1.  Both cases run the
+// fully unrolled body; the test is uniform for the workgroup.  Row-major operands, no K split.
+template <class T, int CB, int RMAX, int U>
+__global__ void __launch_bounds__(wave_kernel_threads(RMAX *CB, U, false)) gemm_wave_balanced_kernel(GemmArgs p) {
+    extern __shared__ f32x4 red[];
+    __shared__ int s_last;
+    const int groups = p.N >> 4;
+    const int rt = blockIdx.x;
+    const int rg0 = (int)((long long)rt * groups / (int)gridDim.x);
+    const int nr = (int)((long long)(rt + 1) * groups / (int)gridDim.x) - rg0;
+    if (nr == RMAX)
+        gemm_wave_body<T, false, CB, RMAX, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR, U, false>(p, rt, 0, rg0, gridDim.x, red, s_last);
+    else
+        gemm_wave_body<T, false, CB, RMAX - 1, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR, U, false>(p, rt, 0, rg0, gridDim.x, red, s_last);
 }
 
 // Kernel 2: row-shared tile kernel (see mlk_tile.cuh).  Four waves per workgroup, R row groups
@@ -484,12 +505,55 @@ static int launch(const GemmArgs &p, hipStream_t s) {
     return MLK_OK;
 }
 
+// What a CU can pull through its vector memory path bounds these kernels when the weight matrix has
+// few rows: with a fixed number of row groups per workgroup the grid of N = 11008 at 16 tokens is 172
+// workgroups, a third of the CUs idle and the others over their share.  Kernel id 4 runs one workgroup
+// per CU instead.
+template <class T, int CB, int RMAX>
+static int launch_balanced(const GemmArgs &p, int wgs, hipStream_t s) {
+    constexpr int U = 4;     // k tiles in flight per wave (measured best at 2 waves per workgroup)
+    GemmArgs q = p;
+    q.SK = 1;
+    while (q.WK * 64 > wave_kernel_threads(RMAX * CB, U, false) || (size_t)q.WK * RMAX * CB * 1024 > 64 * 1024) q.WK >>= 1;
+    size_t lds = q.WK > 1 ? (size_t)q.WK * RMAX * CB * 1024 : 0;
+    gemm_wave_balanced_kernel<T, CB, RMAX, U><<<wgs, q.WK * 64, lds, s>>>(q);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+// number of workgroups for kernel id 4 and the larger of the two row-group counts, or 0 when it does not apply
+static int balanced_grid(const GemmArgs &p, int CB, int *r_max) {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
+        cus = prop.multiProcessorCount;
+    }
+    const int groups = p.N / 16;
+    if (groups <= cus) return 0;
+    const int r = (groups + cus - 1) / cus;
+    if (r < 2 || r > 4 || r * CB > 4) return 0;
+    *r_max = r;
+    return cus;
+}
+
 template <class T, bool FP8, int BMODE, int CMODE>
 static int launch_rc(const GemmArgs &p, int kernel_id, int R, int CB, hipStream_t s) {
 #define MLK_CASE(RR, CC)                                                                        \
     if (R == RR && CB == CC)                                                                    \
         return (kernel_id == 2 && tile_kernel_fits(p, RR, CC)) ? launch_tile<T, FP8, CC, RR, BMODE, CMODE>(p, s) \
                                                           : launch<T, FP8, CC, RR, BMODE, CMODE>(p, s);
+    if constexpr (!FP8 && BMODE == MLK_B_ROWMAJOR && CMODE == MLK_C_ROWMAJOR) {
+        if (kernel_id == 4) {
+            int r_max = 0;
+            const int wgs = p.SK == 1 ? balanced_grid(p, CB, &r_max) : 0;
+            if (wgs && CB == 1 && r_max == 2) return launch_balanced<T, 1, 2>(p, wgs, s);
+            if (wgs && CB == 1 && r_max == 3) return launch_balanced<T, 1, 3>(p, wgs, s);
+            if (wgs && CB == 1 && r_max == 4) return launch_balanced<T, 1, 4>(p, wgs, s);
+            if (wgs && CB == 2 && r_max == 2) return launch_balanced<T, 2, 2>(p, wgs, s);
+        }
+    }
     MLK_CASE(1, 1) MLK_CASE(1, 2) MLK_CASE(1, 3) MLK_CASE(1, 4)
     MLK_CASE(2, 1) MLK_CASE(2, 2) MLK_CASE(2, 3) MLK_CASE(2, 4)
     MLK_CASE(4, 1) MLK_CASE(4, 2) MLK_CASE(4, 3) MLK_CASE(4, 4)

@@ -152,6 +152,9 @@ def scan_gemm(table, shapes, tokens, iters):
             # row-major activations and output)
             if m <= 16 and mode in ("rowmajor", "fp8"):
                 grid += [(10 + u, r, w, sk) for (_, r, w, sk) in list(grid) if _ == 1 for u in (2, 4, 6, 8)]
+            # kernel 4: one workgroup per CU, row groups dealt out evenly (16-bit weights, up to 32 tokens)
+            if mode == "rowmajor" and m <= 32:
+                grid += [(4, 1, w, 1) for w in (1, 2, 4, 8)]
             for kid, p1, p2, p3 in grid:
                 if (n // 16) % p1:
                     continue

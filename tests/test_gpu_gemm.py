@@ -146,6 +146,41 @@ def test_gemm_wide_default_parameters(mlk):
     assert_close(c8, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), bb), RTOL, ATOL, "wide default fp8")
 
 
+@pytest.mark.parametrize("n", [16 * 300, 16 * 384, 16 * 688, 16 * 768, 16 * 1000])
+@pytest.mark.parametrize("m", [1, 7, 16, 32, 40])
+def test_gemm_balanced_rows_kernel(mlk, n, m):
+    """kernelId 4: one workgroup per CU, the row groups dealt out evenly (one to four per workgroup, uneven
+    deals included).  More than 32 tokens, or shapes it does not take, run as kernel 1."""
+    k = 256
+    w = randn((n, k), torch.bfloat16, 0.05, 71)
+    b = randn((m, k), torch.bfloat16, 1.0, 72)
+    bias = randn((1, n), torch.bfloat16, 1.0, 73)
+    a = pack_a(w).cuda()
+    for p2 in (1, 2, 8):
+        c = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=2.0, kernelParam1=1, kernelParam2=p2, kernelParam3=1,
+                                    kernelId=4, bias=bias.cuda())
+        assert_close(c, ogemm.linear_expected(w, b, 2.0, bias), RTOL, ATOL, "balanced rows n=%d m=%d" % (n, m))
+
+
+def test_gemm_balanced_rows_fallbacks(mlk):
+    """Soft-FP8 weights and native operands are outside kernel 4: the id then means kernel 1."""
+    n, k, m = 16 * 300, 512, 16
+    codes = fp8_codes((n - n % 128, k), 81)
+    n8 = codes.shape[0]
+    g = torch.Generator().manual_seed(82)
+    scale = (torch.rand((n8 // 128, k // 128), generator=g) * 0.02 + 0.001).float()
+    b = randn((m, k), torch.bfloat16, 1.0, 83)
+    c = mlk.gemm_layoutA_soft_fp8_wapper(pack_a(codes).cuda(), scale.cuda(), b.cuda(), n8, m, k, kernelParam1=1,
+                                         kernelParam2=4, kernelParam3=1, kernelId=4)
+    assert_close(c, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), b), RTOL, ATOL, "kernel 4 on fp8")
+    w = randn((n, k), torch.float16, 0.05, 84)
+    bh = randn((m, k), torch.float16, 1.0, 85)
+    a = pack_a(w).cuda()
+    c_rm = mlk.gemm_layoutAB_ContinuousC_wapper(a, mlk.layoutB(bh.cuda()), n, m, k, kernelParam1=1, kernelParam2=4,
+                                                kernelParam3=1, kernelId=4)
+    assert_close(c_rm, ogemm.linear_expected(w, bh), RTOL, ATOL, "kernel 4 on native B")
+
+
 def test_gemm_special_cases(mlk):
     n = k = 256
     eye = torch.eye(n, dtype=torch.float16)

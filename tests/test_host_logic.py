@@ -12,6 +12,7 @@ def test_gemm_guard_accepts_both_kernels_and_rejects_bad_rows():
     assert ops._gemm_guard((2, 2, 1, 2), 11008) == (2, 2, 1, 2)
     assert ops._gemm_guard((14, 4, 2, 1), 11008) == (14, 4, 2, 1)    # kernel 1 with an explicit ring depth
     assert ops._gemm_guard((13, 4, 2, 1), 11008) == (1, 1, 4, 1)
+    assert ops._gemm_guard((4, 1, 2, 1), 11008) == (4, 1, 2, 1)      # one workgroup per CU
     assert ops._gemm_guard((18, 8, 4, 1), 28672) == (18, 8, 4, 1)    # eight row groups per wave
     assert ops._gemm_guard((3, 1, 1, 1), 11008) == (1, 1, 4, 1)      # unknown kernel id
     assert ops._gemm_guard((1, 3, 4, 1), 11008) == (1, 1, 4, 1)      # row groups per wave not in {1,2,4}
