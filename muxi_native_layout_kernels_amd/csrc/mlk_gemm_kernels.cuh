@@ -511,7 +511,7 @@ static int launch(const GemmArgs &p, hipStream_t s) {
 // per CU instead.
 template <class T, int CB, int RMAX>
 static int launch_balanced(const GemmArgs &p, int wgs, hipStream_t s) {
-    constexpr int U = 4;     // k tiles in flight per wave (measured best at 2 waves per workgroup)
+    constexpr int U = RMAX * CB <= 4 ? 4 : (RMAX * CB <= 8 ? 3 : 2);     // k tiles in flight per wave
     GemmArgs q = p;
     q.SK = 1;
     while (q.WK * 64 > wave_kernel_threads(RMAX * CB, U, false) || (size_t)q.WK * RMAX * CB * 1024 > 64 * 1024) q.WK >>= 1;
@@ -533,7 +533,7 @@ static int balanced_grid(const GemmArgs &p, int CB, int *r_max) {
     const int groups = p.N / 16;
     if (groups <= cus) return 0;
     const int r = (groups + cus - 1) / cus;
-    if (r < 2 || r > 4 || r * CB > 4) return 0;
+    if (r < 2 || r > 4 || CB > 2) return 0;   // from three token blocks on the row-shared kernel is faster
     *r_max = r;
     return cus;
 }
@@ -548,10 +548,11 @@ static int launch_rc(const GemmArgs &p, int kernel_id, int R, int CB, hipStream_
         if (kernel_id == 4) {
             int r_max = 0;
             const int wgs = p.SK == 1 ? balanced_grid(p, CB, &r_max) : 0;
-            if (wgs && CB == 1 && r_max == 2) return launch_balanced<T, 1, 2>(p, wgs, s);
-            if (wgs && CB == 1 && r_max == 3) return launch_balanced<T, 1, 3>(p, wgs, s);
-            if (wgs && CB == 1 && r_max == 4) return launch_balanced<T, 1, 4>(p, wgs, s);
-            if (wgs && CB == 2 && r_max == 2) return launch_balanced<T, 2, 2>(p, wgs, s);
+#define MLK_BAL(CC, RR) \
+    if (wgs && CB == CC && r_max == RR) return launch_balanced<T, CC, RR>(p, wgs, s);
+            MLK_BAL(1, 2) MLK_BAL(1, 3) MLK_BAL(1, 4)
+            MLK_BAL(2, 2) MLK_BAL(2, 3) MLK_BAL(2, 4)
+#undef MLK_BAL
         }
     }
     MLK_CASE(1, 1) MLK_CASE(1, 2) MLK_CASE(1, 3) MLK_CASE(1, 4)
