@@ -32,6 +32,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
+MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16 (soft-FP8 weights are widened to bf16 before the product)
 MALL_BYTES = 256 << 20
 
 
@@ -164,6 +165,15 @@ def main():
         return dict(name=name, us=us, bytes=algo, gbps=algo / us / 1e3, frac=algo / us / 1e3 / HBM_PEAK_GBPS,
                     params=[kid, p1, p2, p3], copies=len(A), wall=wall)
 
+    def panel_case(name, n, k, kind, m, steps):
+        """Prefill-sized token counts: bound by the matrix cores (or by the weight stream up to ~300 tokens)."""
+        row = gemm_case(name, n, k, kind, m, steps, 3, copies=2)
+        flops = 2.0 * m * n * k
+        row["tflops"] = flops / row["us"] / 1e6
+        row["mfma_frac"] = row["tflops"] / MFMA_PEAK_TFLOPS
+        row["bound"] = "mfma" if flops / (MFMA_PEAK_TFLOPS * 1e6) > row["bytes"] / (HBM_PEAK_GBPS * 1e3) else "hbm"
+        return row
+
     moe_w = {}
 
     def moe_case(name, T, fp8, steps, warmup):
@@ -261,6 +271,20 @@ def main():
             best = max(best, nbytes / us / 1e3)
         return best
 
+    def pack_case(name, e, n, k, steps):
+        """The device step of the checkpoint converter: row-major expert matrices -> layout-A (read + write)."""
+        src = [(torch.randn((e, n, k), generator=gen, device=dev) * 0.02).to(torch.bfloat16) for _ in range(2)]
+        dst = torch.empty((e, n // 16, k // 8, 16, 8), dtype=torch.bfloat16, device=dev)
+
+        def mk(a):
+            def call():
+                _lib.check(lib.mlk_pack_layout_a(a.data_ptr(), dst.data_ptr(), e, n, k, 2,
+                                                 torch.cuda.current_stream().cuda_stream), "pack_layout_a")
+            return call
+        us, wall = run_graph([mk(a) for a in src], steps, 3)
+        algo = 2 * e * n * k * 2
+        return dict(name=name, us=us, bytes=algo, gbps=algo / us / 1e3, frac=algo / us / 1e3 / HBM_PEAK_GBPS, wall=wall)
+
     # ------------------------------------------------------------ headline
     N, K_, M = 11008, 4096, 16
     head = gemm_case("C2 fp16 gemm_layoutA 11008x4096 M=16", N, K_, 0, M, args.steps, args.warmup)
@@ -292,9 +316,16 @@ def main():
             per_config.append(moe_next_case("next: grouped-routing MoE E=256 top-8 H=7168 I=2048 bf16 T=%d" % T, T, 20, 5))
         moe_w.clear()
         torch.cuda.empty_cache()
+        for m in (256, 1024, 4096):
+            per_config.append(panel_case("next: prefill gemm_layoutA fp16 11008x4096 M=%d" % m, N, K_, 0, m, 20))
+        per_config.append(panel_case("next: prefill gemm_layoutA bf16 8192x8192 M=4096", 8192, 8192, 1, 4096, 10))
+        per_config.append(panel_case("next: prefill gemm_layoutA soft-fp8 28672x8192 M=1024", 28672, 8192, 2, 1024, 10))
+        torch.cuda.empty_cache()
+        per_config.append(pack_case("next: checkpoint conversion, pack_layout_a bf16 [8, 28672, 4096]", 8, 28672, 4096, 10))
+        torch.cuda.empty_cache()
         for row in per_config:
             row.pop("wall", None)
-            for key in ("us", "gbps", "frac", "roofline_us", "ratio_to_roofline"):
+            for key in ("us", "gbps", "frac", "roofline_us", "ratio_to_roofline", "tflops", "mfma_frac"):
                 if key in row:
                     row[key] = round(row[key], 4)
 

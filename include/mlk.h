@@ -118,7 +118,7 @@ int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k
 
 /* --------------------------------------------------------------- narrow GeMM
  * C = T(alpha * B . A^T (+ bias[N])), any M >= 1 (in passes over the weights), A in layout-A, MFMA
- * 16x16x32 with fp32 accumulation.
+ * 16x16x32 (32x32x16 in kernel 3) with fp32 accumulation.
  *
  *   b_mode MLK_B_ROWMAJOR, c_mode MLK_C_ROWMAJOR : `gemm_layoutA` / `_wapper`
  *       csrc/gemm_layout_A.cu:684-787 (ffi.cu:43-45, :74-78) and, with
@@ -139,6 +139,13 @@ int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k
  *                shape it does not tile (N/16 not a multiple of 4 p1, or K/32 not a multiple
  *                of 4 p3).  With row-major B and C it takes more than 64 tokens in passes of up
  *                to 128 (p1 limited to 2) instead of 64
+ *   kernel_id 3  panel kernel for prefill-sized token counts (the large-tile `muxi_hgemm_layoutA`
+ *                of the reference, csrc/muxi_hgemm_layoutA.cu:10-217, is its counterpart): one launch
+ *                for any M; a workgroup computes 256 weight rows x 128 tokens with MFMA 32x32x16,
+ *                weights straight from layout-A (two lane swaps per register turn two 16-row tiles
+ *                into the 32-row operand), activations shared through LDS.  Row-major B and C,
+ *                K % 128 == 0, M * K < 2^31; 16-bit and fp8 weights; p1 and p2 are ignored, p3 = K
+ *                slices (useful while 256-row x 128-token panels x p3 stay below the CU count; ignored up to 64 tokens)
  *   kernel_id 4  kernel 1 with one workgroup per CU: the N/16 row groups are dealt out as evenly as
  *                possible, two to four per workgroup (p1 and p3 are ignored).  What one CU can pull
  *                through its memory path bounds these kernels, so for few weight rows an even

@@ -21,6 +21,10 @@ What the columns select on gfx950 (the rows are produced by the scripts in
                 kernelId     1 = wave-tiled MFMA kernel (waves of a workgroup split K)
                              2 = row-shared tile kernel (4 waves share the activations of
                                  each k window through LDS; kernelParam2 is not used)
+                             3 = panel kernel for more than about a hundred tokens (256 weight
+                                 rows x 128 tokens per workgroup, 32x32x16 MFMA, any number of
+                                 tokens in one launch; row-major operands, K % 128 == 0;
+                                 kernelParam1 and kernelParam2 are not used)
                              4 = kernel 1 with one workgroup per CU and the row groups dealt out
                                  evenly, two to four per workgroup (16-bit weights, row-major
                                  operands, up to 32 tokens, N/16 above the CU count; kernelParam1
@@ -127,6 +131,24 @@ def _gemm_default(n, m, k):
     return (1, r, waves, 1)
 
 
+def panel_k_slices(n, m, k, cus=256):
+    """K slices for kernel id 3: as many as keep every workgroup on a CU of its own (a panel is 256 weight
+    rows x 128 tokens), at most four, and at least four 128-wide k windows per slice."""
+    tiles = ((n + 255) // 256) * ((m + 127) // 128)
+    for sk in (4, 2):
+        if tiles * sk <= cus and (k // 128) // sk >= 4:
+            return sk
+    return 1
+
+
+def _gemm_default_rowmajor(n, m, k):
+    """Row-major activations and output: from about a hundred tokens on the product is bound by the matrix
+    cores and the panel kernel (id 3) takes over."""
+    if m > 96 and k % 128 == 0:
+        return (3, 1, 1, panel_k_slices(n, m, k))
+    return _gemm_default(n, m, k)
+
+
 _SELECTORS = {
     # reference getters: csrc/arg_selector.cu:84-87 (layout gemm), :158-161 (continuous C),
     # :236-239 (gemv fp16), :312-315 (layoutA gemm), :389-392 (layoutA soft fp8), :464-467 (soft-fp8 gemv),
@@ -134,9 +156,10 @@ _SELECTORS = {
     "layout_gemm": _Selector("layout_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK, "layout GEMM", _gemm_default),
     "continuous_gemm": _Selector("continuous_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK, "ContinuousC GEMM",
                                  _gemm_default),
-    "layoutA_gemm": _Selector("layoutA_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK, "layoutA GEMM", _gemm_default),
+    "layoutA_gemm": _Selector("layoutA_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK, "layoutA GEMM",
+                              _gemm_default_rowmajor),
     "layoutA_soft_fp8_gemm": _Selector("layoutA_Soft_Fp8_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK,
-                                       "layoutA soft-FP8 GEMM", _gemm_default),
+                                       "layoutA soft-FP8 GEMM", _gemm_default_rowmajor),
     "gemv_fp16": _Selector("layout_gemv_dispatch_arg.csv", 2, GEMV_FALLBACK, "GEMV", _gemv_default),
     "gemv_bf16": _Selector("layout_gemv_bf16_dispatch_arg.csv", 2, GEMV_FALLBACK, "bf16 GEMV", _gemv_default),
     "gemv_soft_fp8": _Selector("layout_gemv_soft_fp8_dispatch_arg.csv", 2, GEMV_FALLBACK, "soft-FP8 GEMV",

@@ -15,6 +15,12 @@ extern template int launch_modes<F16, false>(const GemmArgs &, int, int, int, in
 extern template int launch_modes<BF16, false>(const GemmArgs &, int, int, int, int, int, hipStream_t);
 extern template int launch_modes<BF16, true>(const GemmArgs &, int, int, int, int, int, hipStream_t);
 
+// kernel id 3 (mlk_panel.hip)
+size_t panel_partial_bytes(int m, int n, int sk);
+int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int a_kind, float alpha, const void *bias,
+                 const float *scale, int occ, int sk, void *counters, size_t counter_bytes, void *partial,
+                 size_t partial_bytes, hipStream_t s);
+
 }  // namespace mlk
 
 using namespace mlk;
@@ -30,7 +36,9 @@ extern "C" size_t mlk_gemm_workspace_bytes(int m, int n, int p1, int p3) {
     int cb = (m + 15) / 16;
     if (cb > 8) cb = 8;                                  // kernel 2 takes up to 128 tokens per weight pass
     if (p3 <= 1) return 0;
-    return kCounterBytes + (size_t)p3 * (size_t)(n / 16) * cb * 1024;
+    size_t bytes = (size_t)p3 * (size_t)(n / 16) * cb * 1024;
+    if (m > 64 && panel_partial_bytes(m, n, p3) > bytes) bytes = panel_partial_bytes(m, n, p3);   // kernel id 3 folds whole panels
+    return kCounterBytes + bytes;
 }
 
 extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, int n, int k, int a_kind, int x_kind,
@@ -40,7 +48,7 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
     MLK_REQUIRE(m >= 0 && n >= 0 && k >= 0, "gemm: negative size");
     MLK_REQUIRE(n % 16 == 0, "gemm: N % 16 must be 0");
     MLK_REQUIRE(k % 32 == 0, "gemm: K % 32 must be 0");
-    MLK_REQUIRE(kernel_id == 1 || kernel_id == 2 || kernel_id == 4 || kernel_id == 12 || kernel_id == 14 || kernel_id == 16 ||
+    MLK_REQUIRE(kernel_id == 1 || kernel_id == 2 || kernel_id == 3 || kernel_id == 4 || kernel_id == 12 || kernel_id == 14 || kernel_id == 16 ||
                     kernel_id == 18,
                 "gemm: unknown kernel id");
     MLK_REQUIRE(p1 == 1 || p1 == 2 || p1 == 4 || p1 == 8, "gemm: row groups per wave (p1) must be 1, 2, 4 or 8");
@@ -62,6 +70,16 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
     }
     if (m == 0 || n == 0) return MLK_OK;
     MLK_REQUIRE(a && b && c, "gemm: null pointer");
+    if (kernel_id == 3) {
+        // panel kernel: any number of tokens in one launch; p3 = K slices (one slice up to 64 tokens, where the
+        // workspace is sized for the narrow kernels)
+        MLK_REQUIRE(b_mode == MLK_B_ROWMAJOR && c_mode == MLK_C_ROWMAJOR, "gemm: the panel kernel takes row-major B and C");
+        MLK_REQUIRE(k % 128 == 0, "gemm: the panel kernel needs K % 128 == 0");
+        uint8_t *ws = (uint8_t *)workspace;
+        const size_t part_bytes = workspace_bytes > kCounterBytes ? workspace_bytes - kCounterBytes : 0;
+        return launch_panel(a, b, c, m, n, k, fp8 ? MLK_FP8_E4M3 : x_kind, alpha, bias, scale, p2 >= 2 ? 2 : 1, m > 64 ? p3 : 1, ws, kCounterBytes,
+                            ws ? ws + kCounterBytes : nullptr, ws ? part_bytes : 0, (hipStream_t)stream);
+    }
     int sk = p3;
     if (sk > k / 32) sk = k / 32 > 0 ? k / 32 : 1;
     const int cb_max = (m + 15) / 16 < 8 ? (m + 15) / 16 : 8;

@@ -146,6 +146,62 @@ def test_gemm_wide_default_parameters(mlk):
     assert_close(c8, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), bb), RTOL, ATOL, "wide default fp8")
 
 
+@pytest.mark.parametrize("m", [1, 65, 128, 129, 200, 256, 300, 640])
+@pytest.mark.parametrize("n,k,p3", [(512, 256, 1), (272, 384, 1), (272, 384, 3), (1040, 1024, 2), (256, 128, 4)])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_gemm_panel_kernel(mlk, m, n, k, p3, dtype):
+    """kernelId 3: 256-row x 128-token panels with MFMA 32x32x16; ragged token counts, row counts that are not
+    a multiple of 256 (or of 32: 272 = 17 row groups), K slices that do not divide the windows evenly, one
+    window per slice, more slices than windows."""
+    w = randn((n, k), dtype, 0.05, 91)
+    b = randn((m, k), dtype, 1.0, 92)
+    bias = randn((1, n), dtype, 1.0, 93)
+    a = pack_a(w).cuda()
+    c = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=1, kernelParam2=1, kernelParam3=p3,
+                                kernelId=3, bias=bias.cuda())
+    assert c.shape == (m, n) and c.dtype == dtype
+    assert_close(c, ogemm.linear_expected(w, b, 0.5, bias), RTOL, ATOL, "panel n=%d k=%d M=%d" % (n, k, m))
+    c2 = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=1, kernelParam2=1, kernelParam3=p3,
+                                 kernelId=3, bias=bias.cuda())
+    assert torch.equal(c, c2)
+
+
+@pytest.mark.parametrize("m", [100, 256, 385])
+@pytest.mark.parametrize("scaled", [False, True])
+def test_gemm_panel_kernel_soft_fp8(mlk, m, scaled):
+    n, k = 640, 512
+    codes = fp8_codes((n, k), 95)
+    g = torch.Generator().manual_seed(96)
+    scale = (torch.rand((n // 128, k // 128), generator=g) * 0.02 + 0.001).float() if scaled else None
+    b = randn((m, k), torch.bfloat16, 1.0, 97)
+    for p3 in (1, 2):
+        c = mlk.gemm_layoutA_soft_fp8_wapper(pack_a(codes).cuda(), None if scale is None else scale.cuda(), b.cuda(),
+                                             n, m, k, kernelParam1=1, kernelParam2=1, kernelParam3=p3, kernelId=3)
+        want = ogemm.softfp8_linear_expected(codes.numpy(), None if scale is None else scale.numpy(), b)
+        assert_close(c, want, RTOL, ATOL, "panel fp8 M=%d slices=%d" % (m, p3))
+
+
+def test_gemm_panel_kernel_is_the_wide_default(mlk):
+    """Above about a hundred tokens the heuristic for unscanned shapes picks the panel kernel; a K that is no
+    multiple of 128 keeps the row-shared kernel, and the panel kernel refuses it when asked for by id."""
+    from muxi_native_layout_kernels_amd import arg_selector
+    assert arg_selector.selector("layoutA_gemm").get_args((4096, 300, 1024))[0] == 3
+    assert arg_selector.selector("layoutA_soft_fp8_gemm").get_args((4096, 300, 1024))[0] == 3
+    assert arg_selector.selector("layoutA_gemm").get_args((4096, 300, 1088))[0] == 2
+    assert arg_selector.selector("layout_gemm").get_args((4096, 304, 1024))[0] == 2       # native operands
+    n, k, m = 4096, 1024, 300
+    w = randn((n, k), torch.bfloat16, 0.02, 98)
+    b = randn((m, k), torch.bfloat16, 1.0, 99)
+    c = mlk.gemm_layoutA_linear(pack_a(w).cuda(), b.cuda())
+    assert_close(c, ogemm.linear_expected(w, b), RTOL, ATOL, "panel default")
+    with pytest.raises(RuntimeError, match="K % 128"):
+        mlk.gemm_layoutA_wapper(pack_a(w[:, :960].contiguous()).cuda(), b[:, :960].contiguous().cuda(), n, m, 960,
+                                kernelParam1=1, kernelParam2=1, kernelParam3=1, kernelId=3)
+    with pytest.raises(RuntimeError, match="row-major"):
+        mlk.gemm_layoutABC_wapper(pack_a(w).cuda(), mlk.layoutB(b[:288].contiguous().cuda()), n, 288, k, kernelParam1=1,
+                                  kernelParam2=1, kernelParam3=1, kernelId=3)
+
+
 @pytest.mark.parametrize("n", [16 * 300, 16 * 384, 16 * 688, 16 * 768, 16 * 1000])
 @pytest.mark.parametrize("m", [1, 7, 16, 32, 40])
 def test_gemm_balanced_rows_kernel(mlk, n, m):

@@ -14,7 +14,8 @@ def test_gemm_guard_accepts_both_kernels_and_rejects_bad_rows():
     assert ops._gemm_guard((13, 4, 2, 1), 11008) == (1, 1, 4, 1)
     assert ops._gemm_guard((4, 1, 2, 1), 11008) == (4, 1, 2, 1)      # one workgroup per CU
     assert ops._gemm_guard((18, 8, 4, 1), 28672) == (18, 8, 4, 1)    # eight row groups per wave
-    assert ops._gemm_guard((3, 1, 1, 1), 11008) == (1, 1, 4, 1)      # unknown kernel id
+    assert ops._gemm_guard((3, 1, 1, 2), 11008) == (3, 1, 1, 2)      # panel kernel
+    assert ops._gemm_guard((5, 1, 1, 1), 11008) == (1, 1, 4, 1)      # unknown kernel id
     assert ops._gemm_guard((1, 3, 4, 1), 11008) == (1, 1, 4, 1)      # row groups per wave not in {1,2,4}
     assert ops._gemm_guard((1, 4, 4, 1), 16 * 6) == (1, 1, 4, 1)     # 6 row groups are not a multiple of 4
     assert ops._gemm_guard((1, 1, 5, 1), 4096) == (1, 1, 4, 1)       # waves per workgroup not a power of two
@@ -68,3 +69,20 @@ def test_beta_must_be_zero():
     with pytest.raises(RuntimeError, match="beta"):
         ops._check_beta(0.5)
     ops._check_beta(0)
+
+
+def test_panel_kernel_default_and_k_slices():
+    """Unscanned row-major shapes: the panel kernel from about a hundred tokens on, with as many K slices as
+    keep 256-row x 128-token panels x slices within the CU count."""
+    from muxi_native_layout_kernels_amd import arg_selector as sel
+    assert sel.panel_k_slices(11008, 128, 4096) == 4          # 43 panels
+    assert sel.panel_k_slices(11008, 256, 4096) == 2          # 86 panels
+    assert sel.panel_k_slices(11008, 512, 4096) == 1          # 172 panels
+    assert sel.panel_k_slices(8192, 256, 8192) == 4           # 64 panels
+    assert sel.panel_k_slices(28672, 128, 8192) == 2          # 112 panels
+    assert sel.panel_k_slices(1024, 128, 1024) == 2           # 8 windows: at least four per slice
+    assert sel.panel_k_slices(1024, 128, 384) == 1
+    assert sel._gemm_default_rowmajor(11008, 512, 4096) == (3, 1, 1, 1)
+    assert sel._gemm_default_rowmajor(11008, 96, 4096)[0] == 2      # still the row-shared kernel
+    assert sel._gemm_default_rowmajor(11008, 512, 4096 + 64)[0] == 2  # K is no multiple of 128
+    assert sel._gemm_default(11008, 512, 4096)[0] == 2              # native operands never get the panel kernel
