@@ -24,7 +24,8 @@ What the columns select on gfx950 (the rows are produced by the scripts in
                              3 = panel kernel for more than about a hundred tokens (256 weight
                                  rows x 128 tokens per workgroup, 32x32x16 MFMA, any number of
                                  tokens in one launch; row-major operands, K % 128 == 0;
-                                 kernelParam1 and kernelParam2 are not used)
+                                 kernelParam1 is not used, kernelParam2 = 1: panels of 128
+                                 tokens, 2: of 256 tokens, else chosen from the shape)
                              4 = kernel 1 with one workgroup per CU and the row groups dealt out
                                  evenly, two to four per workgroup (16-bit weights, row-major
                                  operands, up to 32 tokens, N/16 above the CU count; kernelParam1
@@ -145,7 +146,7 @@ def _gemm_default_rowmajor(n, m, k):
     """Row-major activations and output: from about a hundred tokens on the product is bound by the matrix
     cores and the panel kernel (id 3) takes over."""
     if m > 96 and k % 128 == 0:
-        return (3, 1, 1, panel_k_slices(n, m, k))
+        return (3, 1, 4, panel_k_slices(n, m, k))
     return _gemm_default(n, m, k)
 
 

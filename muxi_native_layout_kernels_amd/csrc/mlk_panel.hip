@@ -28,13 +28,14 @@
 
 namespace mlk {
 
+// Two panel shapes: TB = 4 blocks of 32 tokens (128 tokens, k windows of 128) and TB = 8 (256 tokens, k windows
+// of 64).  What a CU can pull through its memory path bounds the kernel once the matrix cores are fed, and a
+// 256 x 256 panel moves a third fewer operand bytes per flop than a 256 x 128 one.
 constexpr int kPanelR = 4;                                   // row groups per wave (two pairs)
-constexpr int kPanelTB = 4;                                  // blocks of 32 tokens per workgroup
-constexpr int kPanelKW = 4;                                  // k tiles per window (128 k)
-constexpr int kPanelTileStride = kPanelTB * 4 * 33 + 4;      // granules between the k tiles of a window
-constexpr int kPanelWin = kPanelKW * kPanelTileStride;       // granules of one LDS window
 constexpr int kPanelRowsPerWg = kTileWaves * kPanelR * 16;   // 256
-constexpr int kPanelTokensPerWg = kPanelTB * 32;             // 128
+__host__ __device__ constexpr int panel_kw(int tb) { return tb == 4 ? 4 : 2; }                 // k tiles per window
+__host__ __device__ constexpr int panel_tile_stride(int tb) { return tb * 4 * 33 + 4; }         // granules between k tiles
+__host__ __device__ constexpr int panel_win(int tb) { return panel_kw(tb) * panel_tile_stride(tb); }
 
 struct PanelArgs {
     const uint8_t *A;
@@ -61,11 +62,11 @@ __device__ __forceinline__ void pair_to_rows32(u32x4 &x, u32x4 &y) {
     }
 }
 
-template <class T, bool FP8, int OCC>
-__global__ void __launch_bounds__(256, OCC) gemm_panel_kernel(PanelArgs p) {
+template <class T, bool FP8, int TB>
+__global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     extern __shared__ u32x4 win[];
     __shared__ int s_last;
-    constexpr int R = kPanelR, TB = kPanelTB, KW = kPanelKW, WG = kPanelWin, TS = kPanelTileStride;
+    constexpr int R = kPanelR, KW = panel_kw(TB), WG = panel_win(TB), TS = panel_tile_stride(TB);
     constexpr int WBYTES = FP8 ? 1 : 2;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -81,7 +82,7 @@ __global__ void __launch_bounds__(256, OCC) gemm_panel_kernel(PanelArgs p) {
 
     const int groups = p.N >> 4;
     const int rg0 = (rt * kTileWaves + wave) * R;
-    const int tok0 = tt * kPanelTokensPerWg;
+    const int tok0 = tt * (TB * 32);
     const int nwin_total = p.K / (KW * 32);
     const int wbeg = (int)((long long)sk * nwin_total / p.SK);
     const int nwin = (int)((long long)(sk + 1) * nwin_total / p.SK) - wbeg;
@@ -97,18 +98,18 @@ __global__ void __launch_bounds__(256, OCC) gemm_panel_kernel(PanelArgs p) {
     ScaleRow srow;
     if (FP8) srow = load_scale_row(p.scale ? p.scale + (size_t)(min(rg0, groups - 1) >> 3) * scale_cols : nullptr, scale_cols, lane);
 
-    // activation staging: a window is 128 tokens x 16 granules; granule i of this thread is token (tid >> 4) + 16 i of
-    // the panel, k granule tid & 15 of the window (k tile colg >> 2, octet colg & 3)
-    constexpr int NG = 8;
-    const int colg = tid & 15;
+    // activation staging: a window is 32 TB tokens x GPR granules (k tile colg >> 2, octet colg & 3); granule i of
+    // this thread is token trow + RP i of the panel, k granule colg
+    constexpr int GPR = KW * 4, RP = 256 / GPR, NG = TB * 32 / RP;
+    const int colg = tid % GPR, trow = tid / GPR;
     uint32_t boff[NG];
 #pragma unroll
     for (int i = 0; i < NG; ++i) {
-        const int tok = min(tok0 + (tid >> 4) + 16 * i, p.M - 1);
+        const int tok = min(tok0 + trow + RP * i, p.M - 1);
         boff[i] = (uint32_t)tok * (uint32_t)p.K + colg * 8;
     }
-    // granule i: token block i >> 1, token (tid >> 4) + 16 (i & 1) of its 32
-    const int st_idx = (colg >> 2) * TS + (colg & 3) * 33 + (tid >> 4);       // + (i >> 1) * 4 * 33 + (i & 1) * 16
+    const int st_idx = (colg >> 2) * TS + (colg & 3) * 33 + trow;             // + st_off(i)
+    auto st_off = [](int i) { return ((RP * i) / 32) * 4 * 33 + (RP * i) % 32; };
     const int ld_idx = (lane >> 5) * 33 + (lane & 31);                        // + t * TS + (tb * 4 + 2 s) * 33
 
     f32x16 acc[2][TB];
@@ -137,10 +138,10 @@ __global__ void __launch_bounds__(256, OCC) gemm_panel_kernel(PanelArgs p) {
     };
     auto stage_store = [&](const u32x4 (&br)[NG], int base) {
 #pragma unroll
-        for (int i = 0; i < NG; ++i) win[base + st_idx + (i >> 1) * 4 * 33 + (i & 1) * 16] = br[i];
+        for (int i = 0; i < NG; ++i) win[base + st_idx + st_off(i)] = br[i];
     };
     WeightFrag<FP8> wf[2][KW][R];
-    float sc[2];                                              // one 128-wide scale block per window
+    float sc[2];                                              // a window lies inside one 128-wide scale block
     auto issue_a = [&](int slot, int w, int t) {              // tile t of window w
         const int tile = (wbeg + w) * KW + t;
 #pragma unroll
@@ -148,7 +149,7 @@ __global__ void __launch_bounds__(256, OCC) gemm_panel_kernel(PanelArgs p) {
             if constexpr (FP8) wf[slot][t][r].v = *reinterpret_cast<const u32x2 *>(abase[r] + (size_t)tile * 512 + lane_off);
             else wf[slot][t][r].v = ld_global_u32x4(abase[r] + (size_t)tile * 1024 + lane_off);
         }
-        if (FP8 && t == KW - 1) sc[slot] = scale_at(srow, wbeg + w);   // after the last use of the slot's previous scale
+        if (FP8 && t == KW - 1) sc[slot] = scale_at(srow, tile >> 2);   // after the last use of the slot's previous scale
     };
     u32x4 b0[TB], b1[TB];
     auto rd = [&](u32x4 (&b)[TB], int base, int t, int s) {
@@ -200,10 +201,12 @@ __global__ void __launch_bounds__(256, OCC) gemm_panel_kernel(PanelArgs p) {
         half(std::integral_constant<int, 1>{}, b1, b0);
         half(std::integral_constant<int, 2>{}, b0, b1);
         half(std::integral_constant<int, 3>{}, b1, b0);
-        half(std::integral_constant<int, 4>{}, b0, b1);
-        half(std::integral_constant<int, 5>{}, b1, b0);
-        half(std::integral_constant<int, 6>{}, b0, b1);
-        half(std::integral_constant<int, 7>{}, b1, b0);
+        if constexpr (KW == 4) {
+            half(std::integral_constant<int, 4>{}, b0, b1);
+            half(std::integral_constant<int, 5>{}, b1, b0);
+            half(std::integral_constant<int, 6>{}, b0, b1);
+            half(std::integral_constant<int, 7>{}, b1, b0);
+        }
         cur = nxt;
     };
     using I0 = std::integral_constant<int, 0>;
@@ -269,7 +272,7 @@ __global__ void __launch_bounds__(256, OCC) gemm_panel_kernel(PanelArgs p) {
     const int tile = rt * p.token_tiles + tt;
     const int tiles = p.row_tiles * p.token_tiles;
     auto part_at = [&](int s, int jj) -> size_t {
-        return ((((size_t)s * tiles + tile) * kTileWaves + wave) * 32 + jj) * 64 + lane;
+        return ((((size_t)s * tiles + tile) * kTileWaves + wave) * (2 * TB * 4) + jj) * 64 + lane;
     };
     // partials travel as agent-scope (write-through / always-miss) accesses, like in the narrow kernels; a release /
     // acquire fence pair around ordinary stores was measured slower (it writes back and invalidates a whole L2)
@@ -295,17 +298,17 @@ __global__ void __launch_bounds__(256, OCC) gemm_panel_kernel(PanelArgs p) {
         for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[pr][tb][e] = 0.f;
-    for (int s = 0; s < p.SK; ++s) {
-        f32x4 t[2 * TB * 4];
 #pragma unroll
-        for (int jj = 0; jj < 2 * TB * 4; ++jj) t[jj] = ld_agent_f32x4(&p.partial[part_at(s, jj)]);
+    for (int pr = 0; pr < 2; ++pr)
+        for (int s = 0; s < p.SK; ++s) {
+            f32x4 t[TB * 4];
 #pragma unroll
-        for (int pr = 0; pr < 2; ++pr)
+            for (int jj = 0; jj < TB * 4; ++jj) t[jj] = ld_agent_f32x4(&p.partial[part_at(s, pr * TB * 4 + jj)]);
 #pragma unroll
             for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
-                for (int e = 0; e < 16; ++e) acc[pr][tb][e] += t[(pr * TB + tb) * 4 + (e >> 2)][e & 3];
-    }
+                for (int e = 0; e < 16; ++e) acc[pr][tb][e] += t[tb * 4 + (e >> 2)][e & 3];
+        }
 #pragma unroll
     for (int pr = 0; pr < 2; ++pr)
 #pragma unroll
@@ -314,15 +317,31 @@ __global__ void __launch_bounds__(256, OCC) gemm_panel_kernel(PanelArgs p) {
             for (int g = 0; g < 4; ++g) epilogue(pr, tb, g, quad(acc[pr][tb], g));
 }
 
-size_t panel_partial_bytes(int m, int n, int sk) {
-    const size_t row_tiles = (n + kPanelRowsPerWg - 1) / kPanelRowsPerWg;
-    const size_t token_tiles = (m + kPanelTokensPerWg - 1) / kPanelTokensPerWg;
-    return (size_t)sk * row_tiles * token_tiles * kPanelRowsPerWg * kPanelTokensPerWg * 4;
+// Tokens per panel when the caller leaves the choice open.  Workgroups run one per CU in rounds, and a 256-token
+// panel takes 1.92 times as long as a 128-token one (measured), so the width with the cheaper sum of rounds wins.
+int panel_tokens(int m, int n) {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0;
+        hipDeviceProp_t prop;
+        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
+        if (cus <= 0) cus = 256;
+    }
+    const long long row_tiles = (n + kPanelRowsPerWg - 1) / kPanelRowsPerWg;
+    const long long rounds128 = (row_tiles * ((m + 127) / 128) + cus - 1) / cus;
+    const long long rounds256 = (row_tiles * ((m + 255) / 256) + cus - 1) / cus;
+    return rounds256 * 192 < rounds128 * 100 ? 256 : 128;
 }
 
-// a_kind: MLK_F16, MLK_BF16 or MLK_FP8_E4M3 (bf16 activations); occ: workgroups per CU the kernel is compiled for
+size_t panel_partial_bytes(int m, int n, int sk) {
+    const size_t row_tiles = (n + kPanelRowsPerWg - 1) / kPanelRowsPerWg;
+    const size_t tokens = (size_t)((m + 255) / 256) * 256;       // covers both panel widths
+    return (size_t)sk * row_tiles * kPanelRowsPerWg * tokens * 4;
+}
+
+// a_kind: MLK_F16, MLK_BF16 or MLK_FP8_E4M3 (bf16 activations); width: tokens per panel (128 or 256), anything else = panel_tokens(m, n)
 int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int a_kind, float alpha, const void *bias,
-                 const float *scale, int occ, int sk, void *counters, size_t counter_bytes, void *partial,
+                 const float *scale, int width, int sk, void *counters, size_t counter_bytes, void *partial,
                  size_t partial_bytes, hipStream_t s) {
     PanelArgs p;
     p.A = (const uint8_t *)a;
@@ -336,11 +355,13 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
     p.N = n;
     p.K = k;
     p.alpha = alpha;
+    if (width != 128 && width != 256) width = panel_tokens(m, n);
     p.row_tiles = (n + kPanelRowsPerWg - 1) / kPanelRowsPerWg;
-    p.token_tiles = (m + kPanelTokensPerWg - 1) / kPanelTokensPerWg;
-    MLK_REQUIRE(k % (kPanelKW * 32) == 0, "gemm: the panel kernel needs K % 128 == 0");
+    p.token_tiles = (m + width - 1) / width;
+    MLK_REQUIRE(k % 128 == 0, "gemm: the panel kernel needs K % 128 == 0");
     MLK_REQUIRE((long long)m * k < (1ll << 31), "gemm: the panel kernel indexes activations with 32 bits");
-    if (sk > k / (kPanelKW * 32)) sk = k / (kPanelKW * 32);
+    const int windows = k / (panel_kw(width / 32) * 32);
+    if (sk > windows) sk = windows;
     if (sk < 1) sk = 1;
     p.SK = sk;
     if (sk > 1) {
@@ -350,23 +371,29 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
         if (partial_bytes < panel_partial_bytes(m, n, sk)) return fail(MLK_ERR_WORKSPACE, "gemm: workspace too small");
     }
     const int grid = ((p.row_tiles + 7) / 8) * 8 * p.token_tiles * sk;
-    const size_t lds = (size_t)3 * kPanelWin * 16;
-    (void)occ;                                             // one workgroup per CU: the register ring and the accumulators take a whole SIMD's file
-    // more than 64 KiB of dynamic LDS has to be requested once per kernel
-#define MLK_PANEL(TT, F8)                                                                                          \
+    // one workgroup per CU (the register ring and the accumulators take a whole SIMD's file); more than 64 KiB of
+    // dynamic LDS has to be requested once per kernel
+#define MLK_PANEL(TT, F8, TBB)                                                                                     \
     do {                                                                                                           \
+        const size_t lds = (size_t)3 * panel_win(TBB) * 16;                                                        \
         static bool ready = false;                                                                                 \
         if (!ready) {                                                                                              \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_panel_kernel<TT, F8, 1>),      \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_panel_kernel<TT, F8, TBB>),    \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);             \
             if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));                                \
             ready = true;                                                                                          \
         }                                                                                                          \
-        gemm_panel_kernel<TT, F8, 1><<<grid, 256, lds, s>>>(p);                                                    \
+        gemm_panel_kernel<TT, F8, TBB><<<grid, 256, lds, s>>>(p);                                                  \
     } while (0)
-    if (a_kind == MLK_FP8_E4M3) MLK_PANEL(BF16, true);
-    else if (a_kind == MLK_F16) MLK_PANEL(F16, false);
-    else MLK_PANEL(BF16, false);
+    if (width == 256) {
+        if (a_kind == MLK_FP8_E4M3) MLK_PANEL(BF16, true, 8);
+        else if (a_kind == MLK_F16) MLK_PANEL(F16, false, 8);
+        else MLK_PANEL(BF16, false, 8);
+    } else {
+        if (a_kind == MLK_FP8_E4M3) MLK_PANEL(BF16, true, 4);
+        else if (a_kind == MLK_F16) MLK_PANEL(F16, false, 4);
+        else MLK_PANEL(BF16, false, 4);
+    }
 #undef MLK_PANEL
     MLK_LAUNCH_CHECK();
     return MLK_OK;

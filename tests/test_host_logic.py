@@ -82,7 +82,7 @@ def test_panel_kernel_default_and_k_slices():
     assert sel.panel_k_slices(28672, 128, 8192) == 2          # 112 panels
     assert sel.panel_k_slices(1024, 128, 1024) == 2           # 8 windows: at least four per slice
     assert sel.panel_k_slices(1024, 128, 384) == 1
-    assert sel._gemm_default_rowmajor(11008, 512, 4096) == (3, 1, 1, 1)
+    assert sel._gemm_default_rowmajor(11008, 512, 4096) == (3, 1, 4, 1)
     assert sel._gemm_default_rowmajor(11008, 96, 4096)[0] == 2      # still the row-shared kernel
     assert sel._gemm_default_rowmajor(11008, 512, 4096 + 64)[0] == 2  # K is no multiple of 128
     assert sel._gemm_default(11008, 512, 4096)[0] == 2              # native operands never get the panel kernel
