@@ -124,8 +124,8 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     // MFMAs (16 k x four token blocks x two row pairs).  While a half step multiplies out of one set of
     // fragment registers the LDS reads of the next half step land in the other set.  Everything that
     // comes from memory is requested well before it is used: the weights of tile t of window j + 2
-    // right after tile t of window j has been multiplied (same registers), the activations of window
-    // j + 2 in the middle of window j; they are written to LDS in the middle of window j + 1 and
+    // once tile t of window j has been multiplied (same registers), the activations of window
+    // j + 2 at the start of window j; they are written to LDS in the middle of window j + 1 and
     // published by the single barrier there, so that the reads of the first half step of window
     // j + 2 can go out during the last half step of window j + 1.  With three LDS buffers that one
     // barrier per window is enough: the buffer written in the middle of window j was last read in
@@ -188,10 +188,18 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
             if (hs < 2 * KW - 1) rd(other, cur, (hs + 1) >> 1, (hs + 1) & 1);
             else if (NEXT) rd(other, nxt, 0, 0);
             if (hs == 0 && NEXT2) stage_load(bring[slot], j + 2);
-            __builtin_amdgcn_sched_barrier(0);
+            if (sh == 0 && t > 0 && NEXT2) issue_a(slot, j + 2, t - 1);   // the registers of tile t - 1 are free again
             mm(a, use, sh);
+            // one scheduling region: the LDS reads and global loads above go out between the MFMAs
+#pragma unroll
+            for (int i = 0; i < TB; ++i) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
+                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // global load
+            }
             __builtin_amdgcn_sched_barrier(0);
-            if (sh == 1 && NEXT2) issue_a(slot, j + 2, t);    // the registers of tile t are free again
+            if (hs == 2 * KW - 1 && NEXT2) issue_a(slot, j + 2, KW - 1);
             if (hs == KW - 1) {
                 if (NEXT) stage_store(bring[slot ^ 1], nxt);
                 __syncthreads();
@@ -318,7 +326,7 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
 }
 
 // Tokens per panel when the caller leaves the choice open.  Workgroups run one per CU in rounds, and a 256-token
-// panel takes 1.92 times as long as a 128-token one (measured), so the width with the cheaper sum of rounds wins.
+// panel takes 1.84 times as long as a 128-token one (measured), so the width with the cheaper sum of rounds wins.
 int panel_tokens(int m, int n) {
     static int cus = 0;
     if (cus == 0) {
@@ -330,7 +338,7 @@ int panel_tokens(int m, int n) {
     const long long row_tiles = (n + kPanelRowsPerWg - 1) / kPanelRowsPerWg;
     const long long rounds128 = (row_tiles * ((m + 127) / 128) + cus - 1) / cus;
     const long long rounds256 = (row_tiles * ((m + 255) / 256) + cus - 1) / cus;
-    return rounds256 * 192 < rounds128 * 100 ? 256 : 128;
+    return rounds256 * 184 < rounds128 * 100 ? 256 : 128;
 }
 
 size_t panel_partial_bytes(int m, int n, int sk) {
