@@ -36,6 +36,29 @@ __global__ void __launch_bounds__(256) layout_a_kernel(const G *__restrict__ src
     }
 }
 
+// The same permutation in whole cache lines, for K % 64 == 0: a wave moves 8 rows x 8 octets, so that on the
+// row-major side every row contributes 8 consecutive granules (a 128-byte line of 16-bit elements) and on the
+// native side every octet contributes rows 8 h .. 8 h + 7 (again a full line); the index arithmetic is done
+// once per wave and per KiB instead of per granule.  task = ((row group) * 2 + h) * K/64 + octet block, the
+// row groups of a batch of matrices counted through.
+template <typename G, bool PACK>
+__global__ void __launch_bounds__(256) layout_a_lines_kernel(const G *__restrict__ src, G *__restrict__ dst, uint32_t tasks,
+                                                             int octets) {
+    const int lane = threadIdx.x & 63;
+    const int oo = lane & 7, rr = lane >> 3;
+    const uint32_t blocks = (uint32_t)octets >> 3;
+    const uint32_t wave = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    for (uint32_t t = wave; t < tasks; t += gridDim.x * 4) {
+        const uint32_t ob = t % blocks, x = t / blocks;
+        const uint32_t h = x & 1;
+        const int64_t rg = x >> 1;
+        const int64_t rm = (rg * 16 + 8 * h + rr) * octets + ob * 8 + oo;
+        const int64_t nat = (rg * octets + ob * 8 + oo) * 16 + 8 * h + rr;
+        if (PACK) dst[nat] = src[rm];
+        else dst[rm] = src[nat];
+    }
+}
+
 // layout-B / layout-C: native granule ((c * M/16 + g) * 64 + 16 q + r) <-> row-major
 // granule (16 g + r) * K/8 + 4 c + q.  PACK: row-major -> native (layoutB);
 // !PACK: native -> row-major (reLayoutC).  The thread index always runs over
@@ -138,6 +161,19 @@ static int layout_a_common(const void *src, void *dst, int64_t batch, int n, int
     if (total == 0) return MLK_OK;
     MLK_REQUIRE(src && dst, "layout-A: null pointer");
     hipStream_t s = (hipStream_t)stream;
+    const int64_t tasks = total / 64;
+    if ((k / 8) % 8 == 0 && tasks < (int64_t)1 << 31) {
+        int grid = grid_for(tasks * 64);
+        if (elem_size == 2) {
+            if (pack) layout_a_lines_kernel<uint4, true><<<grid, 256, 0, s>>>((const uint4 *)src, (uint4 *)dst, (uint32_t)tasks, k / 8);
+            else layout_a_lines_kernel<uint4, false><<<grid, 256, 0, s>>>((const uint4 *)src, (uint4 *)dst, (uint32_t)tasks, k / 8);
+        } else {
+            if (pack) layout_a_lines_kernel<uint2, true><<<grid, 256, 0, s>>>((const uint2 *)src, (uint2 *)dst, (uint32_t)tasks, k / 8);
+            else layout_a_lines_kernel<uint2, false><<<grid, 256, 0, s>>>((const uint2 *)src, (uint2 *)dst, (uint32_t)tasks, k / 8);
+        }
+        MLK_LAUNCH_CHECK();
+        return MLK_OK;
+    }
     int grid = grid_for(total);
     if (elem_size == 2) {
         if (pack) layout_a_kernel<uint4, true><<<grid, 256, 0, s>>>((const uint4 *)src, (uint4 *)dst, total, n, k / 8);
