@@ -379,12 +379,15 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
         if (partial_bytes < panel_partial_bytes(m, n, sk)) return fail(MLK_ERR_WORKSPACE, "gemm: workspace too small");
     }
     const int grid = ((p.row_tiles + 7) / 8) * 8 * p.token_tiles * sk;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
     // one workgroup per CU (the register ring and the accumulators take a whole SIMD's file); more than 64 KiB of
     // dynamic LDS has to be requested once per kernel
 #define MLK_PANEL(TT, F8, TBB)                                                                                     \
     do {                                                                                                           \
         const size_t lds = (size_t)3 * panel_win(TBB) * 16;                                                        \
-        static bool ready = false;                                                                                 \
+        static bool ready_on[64] = {};                           /* the attribute belongs to a device */          \
+        bool &ready = ready_on[dev & 63];                                                                          \
         if (!ready) {                                                                                              \
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_panel_kernel<TT, F8, TBB>),    \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);             \
