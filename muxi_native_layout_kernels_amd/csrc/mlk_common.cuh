@@ -165,23 +165,42 @@ __device__ __forceinline__ float lane_xor(float v, int mask) {
 // Partial sums exchanged between workgroups of one kernel.  The L2 caches of the eight XCDs are
 // not coherent with each other for ordinary accesses; agent-scope atomic accesses are (they are
 // issued write-through / always-miss), and unlike an agent-scope fence they do not write back or
-// invalidate a whole L2.  64-bit relaxed atomics carry two floats each.
-__device__ __forceinline__ void st_agent_f32x4(f32x4 *p, f32x4 v) {
-    uint64_t *q = reinterpret_cast<uint64_t *>(p);
+// invalidate a whole L2.  64-bit relaxed atomics carry two floats each.  A tile of `cells` quads is
+// kept as two planes of 8-byte halves (cell i at [i] and [cells + i]), so that the lanes of one
+// access instruction cover whole cache lines; 16 bytes per lane side by side would leave every
+// instruction writing half of each line it touches.
+__device__ __forceinline__ void st_agent_planar(f32x4 *tile, int cells, int i, f32x4 v) {
+    uint64_t *q = reinterpret_cast<uint64_t *>(tile);
     uint64_t lo = (uint64_t)__float_as_uint(v[0]) | ((uint64_t)__float_as_uint(v[1]) << 32);
     uint64_t hi = (uint64_t)__float_as_uint(v[2]) | ((uint64_t)__float_as_uint(v[3]) << 32);
-    __hip_atomic_store(q, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    __hip_atomic_store(q + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(q + i, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(q + cells + i, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ f32x4 ld_agent_f32x4(const f32x4 *p) {
-    const uint64_t *q = reinterpret_cast<const uint64_t *>(p);
-    uint64_t lo = __hip_atomic_load(q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    uint64_t hi = __hip_atomic_load(q + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ f32x4 ld_agent_planar(const f32x4 *tile, int cells, int i) {
+    const uint64_t *q = reinterpret_cast<const uint64_t *>(tile);
+    uint64_t lo = __hip_atomic_load(q + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    uint64_t hi = __hip_atomic_load(q + cells + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     f32x4 v;
     v[0] = __uint_as_float((uint32_t)lo);
     v[1] = __uint_as_float((uint32_t)(lo >> 32));
     v[2] = __uint_as_float((uint32_t)hi);
     v[3] = __uint_as_float((uint32_t)(hi >> 32));
+    return v;
+}
+// Sum of cell i over `n` slices in slice order; `tile_of(s)` is slice s's tile.  The loads of up to
+// eight slices are in flight together (they bypass the caches: a round trip each if issued one by one).
+template <class TileOf>
+__device__ __forceinline__ f32x4 fold_agent_planar(TileOf tile_of, int n, int cells, int i) {
+    f32x4 v = {0.f, 0.f, 0.f, 0.f};
+    for (int s0 = 0; s0 < n; s0 += 8) {
+        f32x4 t[8];
+#pragma unroll
+        for (int s = 0; s < 8; ++s)
+            if (s0 + s < n) t[s] = ld_agent_planar(tile_of(s0 + s), cells, i);
+#pragma unroll
+        for (int s = 0; s < 8; ++s)
+            if (s0 + s < n) v += t[s];
+    }
     return v;
 }
 

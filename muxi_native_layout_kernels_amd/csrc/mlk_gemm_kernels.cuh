@@ -267,7 +267,8 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
         store4<T>(p.C + off, o[0], o[1], o[2], o[3]);
     };
     f32x4 *part = reinterpret_cast<f32x4 *>(p.partial);
-    auto part_at = [&](int s, int j) -> size_t { return (((size_t)s * row_tiles + rt) * NTILE + j) * 64 + lane; };
+    // 64-lane group of accumulator tile j in slice s (two planes of 8-byte halves, see st_agent_planar)
+    auto group_at = [&](int s, int j) -> f32x4 * { return part + (((size_t)s * row_tiles + rt) * NTILE + j) * 64; };
 
     if (p.WK == 1) {
         // a single wave: tiles stay in registers
@@ -281,7 +282,7 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
 #pragma unroll
         for (int r = 0; r < R; ++r)
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) st_agent_f32x4(&part[part_at(sk, r * CB + cb)], acc[r][cb]);
+            for (int cb = 0; cb < CB; ++cb) st_agent_planar(group_at(sk, r * CB + cb), 64, lane, acc[r][cb]);
     } else {
         // fold the WK waves through LDS in wave order; wave w then owns tiles j = w, w + WK, ...
 #pragma unroll
@@ -293,7 +294,7 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
             f32x4 v = red[j * 64 + lane];
             for (int w = 1; w < p.WK; ++w) v += red[(w * NTILE + j) * 64 + lane];
             if (p.SK == 1) epilogue(j, v);
-            else st_agent_f32x4(&part[part_at(sk, j)], v);
+            else st_agent_planar(group_at(sk, j), 64, lane, v);
         }
         if (p.SK == 1) return;
     }
@@ -313,9 +314,7 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
     __syncthreads();
     if (!s_last) return;
     for (int j = wave; j < NTILE; j += p.WK) {
-        f32x4 v = {0.f, 0.f, 0.f, 0.f};
-        for (int s = 0; s < p.SK; ++s) v += ld_agent_f32x4(&part[part_at(s, j)]);
-        epilogue(j, v);
+        epilogue(j, fold_agent_planar([&](int s) { return group_at(s, j); }, p.SK, 64, lane));
     }
 }
 
@@ -425,13 +424,13 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(GemmArgs p) {
         return;
     }
     f32x4 *part = reinterpret_cast<f32x4 *>(p.partial);
-    auto part_at = [&](int s, int j) -> size_t {
-        return ((((size_t)s * row_tiles + rt) * kTileWaves + wave) * NTILE + j) * 64 + lane;
+    auto group_at = [&](int s, int j) -> f32x4 * {
+        return part + ((((size_t)s * row_tiles + rt) * kTileWaves + wave) * NTILE + j) * 64;
     };
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int cb = 0; cb < CB; ++cb) st_agent_f32x4(&part[part_at(sk, r * CB + cb)], acc[r][cb]);
+        for (int cb = 0; cb < CB; ++cb) st_agent_planar(group_at(sk, r * CB + cb), 64, lane, acc[r][cb]);
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -445,9 +444,7 @@ __global__ void __launch_bounds__(256) gemm_tile_kernel(GemmArgs p) {
     for (int r = 0; r < R; ++r)
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) {
-            f32x4 v = {0.f, 0.f, 0.f, 0.f};
-            for (int s = 0; s < p.SK; ++s) v += ld_agent_f32x4(&part[part_at(s, r * CB + cb)]);
-            epilogue(r, cb, v);
+            epilogue(r, cb, fold_agent_planar([&](int s) { return group_at(s, r * CB + cb); }, p.SK, 64, lane));
         }
 }
 

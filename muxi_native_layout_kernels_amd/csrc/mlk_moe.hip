@@ -751,7 +751,7 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
     f32x4 *part = reinterpret_cast<f32x4 *>(p.part);
     auto tile_at = [&](int sk) { return part + ((size_t)sk * gridDim.x + blockIdx.x) * cells; };
     for (int i = threadIdx.x; i < cells; i += blockDim.x)
-        st_agent_f32x4(tile_at(blockIdx.y) + i, *reinterpret_cast<const f32x4 *>(ytile + 4 * i));
+        st_agent_planar(tile_at(blockIdx.y), cells, i, *reinterpret_cast<const f32x4 *>(ytile + 4 * i));
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -761,8 +761,7 @@ __global__ void __launch_bounds__(max_threads_for_tiles(R *CB)) moe_down_kernel(
     __syncthreads();
     if (!s_last) return;
     for (int i = threadIdx.x; i < cells; i += blockDim.x) {
-        f32x4 v = {0.f, 0.f, 0.f, 0.f};
-        for (int sk = 0; sk < (int)gridDim.y; ++sk) v += ld_agent_f32x4(tile_at(sk) + i);
+        const f32x4 v = fold_agent_planar(tile_at, (int)gridDim.y, cells, i);
         const int e = 4 * i, tok = e / yrows, row = e - tok * yrows;
         store4<T>(p.Y + (size_t)tok * p.H + rg0 * 16 + row, v[0], v[1], v[2], v[3]);
     }

@@ -279,8 +279,9 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     }
     const int tile = rt * p.token_tiles + tt;
     const int tiles = p.row_tiles * p.token_tiles;
-    auto part_at = [&](int s, int jj) -> size_t {
-        return ((((size_t)s * tiles + tile) * kTileWaves + wave) * (2 * TB * 4) + jj) * 64 + lane;
+    // 64-lane group of quad jj of this wave in slice s (two planes of 8-byte halves, see st_agent_planar)
+    auto group_at = [&](int s, int jj) -> f32x4 * {
+        return p.partial + ((((size_t)s * tiles + tile) * kTileWaves + wave) * (2 * TB * 4) + jj) * 64;
     };
     // partials travel as agent-scope (write-through / always-miss) accesses, like in the narrow kernels; a release /
     // acquire fence pair around ordinary stores was measured slower (it writes back and invalidates a whole L2)
@@ -289,7 +290,7 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
 #pragma unroll
         for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) st_agent_f32x4(&p.partial[part_at(sk, (pr * TB + tb) * 4 + g)], quad(acc[pr][tb], g));
+            for (int g = 0; g < 4; ++g) st_agent_planar(group_at(sk, (pr * TB + tb) * 4 + g), 64, lane, quad(acc[pr][tb], g));
     __builtin_amdgcn_s_waitcnt(0);
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -299,24 +300,35 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     }
     __syncthreads();
     if (!s_last) return;
-    // slice order; all loads of a slice are in flight together (the accumulator registers take the sums)
+    // slice order; the loads of the next slice are in flight while the current one is added (a round trip to
+    // memory per slice would otherwise be paid in full: these loads bypass the caches)
 #pragma unroll
-    for (int pr = 0; pr < 2; ++pr)
+    for (int pr = 0; pr < 2; ++pr) {
 #pragma unroll
         for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[pr][tb][e] = 0.f;
+        f32x4 t0[TB * 4], t1[TB * 4];
+        auto fetch = [&](f32x4 (&t)[TB * 4], int sl) {
 #pragma unroll
-    for (int pr = 0; pr < 2; ++pr)
-        for (int s = 0; s < p.SK; ++s) {
-            f32x4 t[TB * 4];
-#pragma unroll
-            for (int jj = 0; jj < TB * 4; ++jj) t[jj] = ld_agent_f32x4(&p.partial[part_at(s, pr * TB * 4 + jj)]);
+            for (int jj = 0; jj < TB * 4; ++jj) t[jj] = ld_agent_planar(group_at(sl, pr * TB * 4 + jj), 64, lane);
+        };
+        auto add = [&](const f32x4 (&t)[TB * 4]) {
 #pragma unroll
             for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
                 for (int e = 0; e < 16; ++e) acc[pr][tb][e] += t[tb * 4 + (e >> 2)][e & 3];
+        };
+        fetch(t0, 0);
+        for (int sl = 0; sl < p.SK; sl += 2) {
+            if (sl + 1 < p.SK) fetch(t1, sl + 1);
+            add(t0);
+            if (sl + 1 < p.SK) {
+                if (sl + 2 < p.SK) fetch(t0, sl + 2);
+                add(t1);
+            }
         }
+    }
 #pragma unroll
     for (int pr = 0; pr < 2; ++pr)
 #pragma unroll
