@@ -316,7 +316,7 @@ def main():
             per_config.append(moe_next_case("next: grouped-routing MoE E=256 top-8 H=7168 I=2048 bf16 T=%d" % T, T, 20, 5))
         moe_w.clear()
         torch.cuda.empty_cache()
-        for m in (256, 1024, 4096):
+        for m in (128, 256, 1024, 4096):
             per_config.append(panel_case("next: prefill gemm_layoutA fp16 11008x4096 M=%d" % m, N, K_, 0, m, 20))
         per_config.append(panel_case("next: prefill gemm_layoutA bf16 8192x8192 M=4096", 8192, 8192, 1, 4096, 10))
         per_config.append(panel_case("next: prefill gemm_layoutA soft-fp8 28672x8192 M=1024", 28672, 8192, 2, 1024, 10))

@@ -144,8 +144,9 @@ int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k
  *                for any M; a workgroup computes 256 weight rows x 128 tokens with MFMA 32x32x16,
  *                weights straight from layout-A (two lane swaps per register turn two 16-row tiles
  *                into the 32-row operand), activations shared through LDS.  Row-major B and C,
- *                K % 128 == 0, M * K < 2^31; 16-bit and fp8 weights; p1 is ignored; p2 = 1: panels of 128
- *                tokens, 2: 256 rows x 256 tokens, any other value: chosen from the shape; p3 = K
+ *                K % 128 == 0, M * K < 2^31; 16-bit and fp8 weights; p1 = 2: panels of 128 rows (with 128
+ *                tokens), 4: of 256 rows; p2 = 1: panels of 128 tokens, 2: 256 rows x 256 tokens; any other
+ *                value of p1 or p2: chosen from the shape; p3 = K
  *                slices (useful while 256-row x 128-token panels x p3 stay below the CU count; ignored up to 64 tokens)
  *   kernel_id 4  kernel 1 with one workgroup per CU: the N/16 row groups are dealt out as evenly as
  *                possible, two to four per workgroup (p1 and p3 are ignored).  What one CU can pull

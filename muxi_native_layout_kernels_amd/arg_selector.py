@@ -24,8 +24,9 @@ What the columns select on gfx950 (the rows are produced by the scripts in
                              3 = panel kernel for more than about a hundred tokens (256 weight
                                  rows x 128 tokens per workgroup, 32x32x16 MFMA, any number of
                                  tokens in one launch; row-major operands, K % 128 == 0;
-                                 kernelParam1 is not used, kernelParam2 = 1: panels of 128
-                                 tokens, 2: of 256 tokens, else chosen from the shape)
+                                 kernelParam1 = 2: panels of 128 rows, 4: of 256 rows,
+                                 kernelParam2 = 1: panels of 128 tokens, 2: of 256 tokens,
+                                 other values: chosen from the shape)
                              4 = kernel 1 with one workgroup per CU and the row groups dealt out
                                  evenly, two to four per workgroup (16-bit weights, row-major
                                  operands, up to 32 tokens, N/16 above the CU count; kernelParam1
@@ -132,21 +133,27 @@ def _gemm_default(n, m, k):
     return (1, r, waves, 1)
 
 
-def panel_k_slices(n, m, k, cus=256):
-    """K slices for kernel id 3: as many as keep every workgroup on a CU of its own (a panel is 256 weight
-    rows x 128 tokens), at most four, and at least four 128-wide k windows per slice."""
-    tiles = ((n + 255) // 256) * ((m + 127) // 128)
+def panel_shape(n, m, k, cus=256):
+    """(row groups per wave, K slices) for kernel id 3.  A panel is 256 weight rows x 128 tokens; while there are
+    at most three eighths as many of them as CUs, 128-row panels (two row groups per wave) put twice as many CUs
+    to work.  K slices: as many (4, 2 or 1) as keep every workgroup on a CU of its own, with at least four
+    128-wide k windows per slice."""
+    panels = ((n + 255) // 256) * ((m + 127) // 128)
+    rg = 4
+    if panels * 8 <= cus * 3:
+        rg, panels = 2, ((n + 127) // 128) * ((m + 127) // 128)
     for sk in (4, 2):
-        if tiles * sk <= cus and (k // 128) // sk >= 4:
-            return sk
-    return 1
+        if panels * sk <= cus and (k // 128) // sk >= 4:
+            return rg, sk
+    return rg, 1
 
 
 def _gemm_default_rowmajor(n, m, k):
     """Row-major activations and output: from about a hundred tokens on the product is bound by the matrix
-    cores and the panel kernel (id 3) takes over."""
+    cores and the panel kernel (id 3) takes over (panel width left to the library)."""
     if m > 96 and k % 128 == 0:
-        return (3, 1, 4, panel_k_slices(n, m, k))
+        rg, sk = panel_shape(n, m, k)
+        return (3, rg, 4, sk)
     return _gemm_default(n, m, k)
 
 

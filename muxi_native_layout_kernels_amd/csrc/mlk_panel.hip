@@ -31,8 +31,7 @@ namespace mlk {
 // Two panel shapes: TB = 4 blocks of 32 tokens (128 tokens, k windows of 128) and TB = 8 (256 tokens, k windows
 // of 64).  What a CU can pull through its memory path bounds the kernel once the matrix cores are fed, and a
 // 256 x 256 panel moves a third fewer operand bytes per flop than a 256 x 128 one.
-constexpr int kPanelR = 4;                                   // row groups per wave (two pairs)
-constexpr int kPanelRowsPerWg = kTileWaves * kPanelR * 16;   // 256
+constexpr int kPanelRowsPerWg = kTileWaves * 4 * 16;         // 256 rows: two pairs of row groups per wave (128 with one pair)
 __host__ __device__ constexpr int panel_kw(int tb) { return tb == 4 ? 4 : 2; }                 // k tiles per window
 __host__ __device__ constexpr int panel_tile_stride(int tb) { return tb * 4 * 33 + 4; }         // granules between k tiles
 __host__ __device__ constexpr int panel_win(int tb) { return panel_kw(tb) * panel_tile_stride(tb); }
@@ -62,11 +61,11 @@ __device__ __forceinline__ void pair_to_rows32(u32x4 &x, u32x4 &y) {
     }
 }
 
-template <class T, bool FP8, int TB>
+template <class T, bool FP8, int TB, int PR>
 __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     extern __shared__ u32x4 win[];
     __shared__ int s_last;
-    constexpr int R = kPanelR, KW = panel_kw(TB), WG = panel_win(TB), TS = panel_tile_stride(TB);
+    constexpr int R = 2 * PR, KW = panel_kw(TB), WG = panel_win(TB), TS = panel_tile_stride(TB);   // PR pairs of row groups per wave
     constexpr int WBYTES = FP8 ? 1 : 2;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -112,9 +111,9 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     auto st_off = [](int i) { return ((RP * i) / 32) * 4 * 33 + (RP * i) % 32; };
     const int ld_idx = (lane >> 5) * 33 + (lane & 31);                        // + t * TS + (tb * 4 + 2 s) * 33
 
-    f32x16 acc[2][TB];
+    f32x16 acc[PR][TB];
 #pragma unroll
-    for (int pr = 0; pr < 2; ++pr)
+    for (int pr = 0; pr < PR; ++pr)
 #pragma unroll
         for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
@@ -163,7 +162,7 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
 #pragma unroll
         for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
-            for (int pr = 0; pr < 2; ++pr) {
+            for (int pr = 0; pr < PR; ++pr) {
                 acc[pr][tb] = T::mfma32(a[2 * pr + s], b[tb], acc[pr][tb]);
             }
     };
@@ -173,7 +172,7 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
         for (int r = 0; r < R; ++r) s4[r] = FP8 ? sc[slot] : 1.f;
         weight_operands<FP8, R>(a, wf[slot][t], s4);
         pair_to_rows32(a[0], a[1]);
-        pair_to_rows32(a[2], a[3]);
+        if constexpr (PR == 2) pair_to_rows32(a[2], a[3]);
     };
     int cur = 0;                                              // LDS granule offset of the current window's buffer
     // SLOT: weight slot; NEXT / NEXT2: windows j + 1 / j + 2 exist (compile-time, so the steady loop has no tests)
@@ -270,7 +269,7 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     auto quad = [&](const f32x16 &v, int g) { return f32x4{v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3]}; };
     if (p.SK == 1) {
 #pragma unroll
-        for (int pr = 0; pr < 2; ++pr)
+        for (int pr = 0; pr < PR; ++pr)
 #pragma unroll
             for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
@@ -281,12 +280,12 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     const int tiles = p.row_tiles * p.token_tiles;
     // 64-lane group of quad jj of this wave in slice s (two planes of 8-byte halves, see st_agent_planar)
     auto group_at = [&](int s, int jj) -> f32x4 * {
-        return p.partial + ((((size_t)s * tiles + tile) * kTileWaves + wave) * (2 * TB * 4) + jj) * 64;
+        return p.partial + ((((size_t)s * tiles + tile) * kTileWaves + wave) * (PR * TB * 4) + jj) * 64;
     };
     // partials travel as agent-scope (write-through / always-miss) accesses, like in the narrow kernels; a release /
     // acquire fence pair around ordinary stores was measured slower (it writes back and invalidates a whole L2)
 #pragma unroll
-    for (int pr = 0; pr < 2; ++pr)
+    for (int pr = 0; pr < PR; ++pr)
 #pragma unroll
         for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
@@ -303,7 +302,7 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     // slice order; the loads of the next slice are in flight while the current one is added (a round trip to
     // memory per slice would otherwise be paid in full: these loads bypass the caches)
 #pragma unroll
-    for (int pr = 0; pr < 2; ++pr) {
+    for (int pr = 0; pr < PR; ++pr) {
 #pragma unroll
         for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
@@ -330,7 +329,7 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
         }
     }
 #pragma unroll
-    for (int pr = 0; pr < 2; ++pr)
+    for (int pr = 0; pr < PR; ++pr)
 #pragma unroll
         for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
@@ -359,9 +358,11 @@ size_t panel_partial_bytes(int m, int n, int sk) {
     return (size_t)sk * row_tiles * kPanelRowsPerWg * tokens * 4;
 }
 
-// a_kind: MLK_F16, MLK_BF16 or MLK_FP8_E4M3 (bf16 activations); width: tokens per panel (128 or 256), anything else = panel_tokens(m, n)
+// a_kind: MLK_F16, MLK_BF16 or MLK_FP8_E4M3 (bf16 activations); width: tokens per panel (128 or 256), anything else =
+// panel_tokens(m, n); rows: weight rows per panel (128 or 256; 128 only with 128 tokens), anything else = chosen
+// from the number of panels
 int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int a_kind, float alpha, const void *bias,
-                 const float *scale, int width, int sk, void *counters, size_t counter_bytes, void *partial,
+                 const float *scale, int width, int rows, int sk, void *counters, size_t counter_bytes, void *partial,
                  size_t partial_bytes, hipStream_t s) {
     PanelArgs p;
     p.A = (const uint8_t *)a;
@@ -376,7 +377,6 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
     p.K = k;
     p.alpha = alpha;
     if (width != 128 && width != 256) width = panel_tokens(m, n);
-    p.row_tiles = (n + kPanelRowsPerWg - 1) / kPanelRowsPerWg;
     p.token_tiles = (m + width - 1) / width;
     MLK_REQUIRE(k % 128 == 0, "gemm: the panel kernel needs K % 128 == 0");
     MLK_REQUIRE((long long)m * k < (1ll << 31), "gemm: the panel kernel indexes activations with 32 bits");
@@ -384,6 +384,19 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
     if (sk > windows) sk = windows;
     if (sk < 1) sk = 1;
     p.SK = sk;
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+    if (width == 256) rows = 256;
+    if (rows != 128 && rows != 256) {
+        int cus = 256;
+        hipDeviceProp_t prop;
+        if (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) cus = prop.multiProcessorCount;
+        // few panels: 128-row panels put twice as many CUs to work (a 128-row panel takes two thirds of the time of
+        // a 256-row one); from three eighths of the CU count on, 256-row panels and K slices fill the chip better
+        const long long panels256 = (long long)((n + 255) / 256) * p.token_tiles;
+        rows = panels256 * 8 <= (long long)cus * 3 ? 128 : 256;
+    }
+    p.row_tiles = (n + rows - 1) / rows;
     if (sk > 1) {
         MLK_REQUIRE(partial != nullptr && counters != nullptr, "gemm: a K split across workgroups needs a workspace");
         MLK_REQUIRE((size_t)p.row_tiles * p.token_tiles * sizeof(int) <= counter_bytes,
@@ -391,31 +404,33 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
         if (partial_bytes < panel_partial_bytes(m, n, sk)) return fail(MLK_ERR_WORKSPACE, "gemm: workspace too small");
     }
     const int grid = ((p.row_tiles + 7) / 8) * 8 * p.token_tiles * sk;
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) dev = 0;
     // one workgroup per CU (the register ring and the accumulators take a whole SIMD's file); more than 64 KiB of
     // dynamic LDS has to be requested once per kernel
-#define MLK_PANEL(TT, F8, TBB)                                                                                     \
+#define MLK_PANEL(TT, F8, TBB, PRR)                                                                                    \
     do {                                                                                                           \
         const size_t lds = (size_t)3 * panel_win(TBB) * 16;                                                        \
         static bool ready_on[64] = {};                           /* the attribute belongs to a device */          \
         bool &ready = ready_on[dev & 63];                                                                          \
         if (!ready) {                                                                                              \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_panel_kernel<TT, F8, TBB>),    \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_panel_kernel<TT, F8, TBB, PRR>),    \
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);             \
             if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));                                \
             ready = true;                                                                                          \
         }                                                                                                          \
-        gemm_panel_kernel<TT, F8, TBB><<<grid, 256, lds, s>>>(p);                                                  \
+        gemm_panel_kernel<TT, F8, TBB, PRR><<<grid, 256, lds, s>>>(p);                                                  \
     } while (0)
     if (width == 256) {
-        if (a_kind == MLK_FP8_E4M3) MLK_PANEL(BF16, true, 8);
-        else if (a_kind == MLK_F16) MLK_PANEL(F16, false, 8);
-        else MLK_PANEL(BF16, false, 8);
+        if (a_kind == MLK_FP8_E4M3) MLK_PANEL(BF16, true, 8, 2);
+        else if (a_kind == MLK_F16) MLK_PANEL(F16, false, 8, 2);
+        else MLK_PANEL(BF16, false, 8, 2);
+    } else if (rows == 256) {
+        if (a_kind == MLK_FP8_E4M3) MLK_PANEL(BF16, true, 4, 2);
+        else if (a_kind == MLK_F16) MLK_PANEL(F16, false, 4, 2);
+        else MLK_PANEL(BF16, false, 4, 2);
     } else {
-        if (a_kind == MLK_FP8_E4M3) MLK_PANEL(BF16, true, 4);
-        else if (a_kind == MLK_F16) MLK_PANEL(F16, false, 4);
-        else MLK_PANEL(BF16, false, 4);
+        if (a_kind == MLK_FP8_E4M3) MLK_PANEL(BF16, true, 4, 1);
+        else if (a_kind == MLK_F16) MLK_PANEL(F16, false, 4, 1);
+        else MLK_PANEL(BF16, false, 4, 1);
     }
 #undef MLK_PANEL
     MLK_LAUNCH_CHECK();

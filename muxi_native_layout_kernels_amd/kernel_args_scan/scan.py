@@ -155,11 +155,11 @@ def scan_gemm(table, shapes, tokens, iters):
             # kernel 4: one workgroup per CU, row groups dealt out evenly (16-bit weights, up to 32 tokens)
             if mode == "rowmajor" and m <= 32:
                 grid += [(4, 1, w, 1) for w in (1, 2, 4, 8)]
-            # kernel 3: panels of 256 rows x 128 / 256 tokens (row-major operands, K % 128 == 0); above 64 tokens the
+            # kernel 3: panels of 128 / 256 rows x 128 / 256 tokens (row-major operands, K % 128 == 0); above 64 tokens the
             # wave kernel is out of the race
             if mode in ("rowmajor", "fp8") and m > 64 and k % 128 == 0:
                 grid = [g for g in grid if g[0] != 1]
-                grid += [(3, 1, w, sk) for w in (1, 2) for sk in (1, 2, 4) if (k // 128) // sk >= 2]
+                grid += [(3, rg, w, sk) for rg, w in ((2, 1), (4, 1), (4, 2)) for sk in (1, 2, 4) if (k // 128) // sk >= 2]
             for kid, p1, p2, p3 in grid:
                 if (n // 16) % p1:
                     continue

@@ -157,12 +157,13 @@ def test_gemm_panel_kernel(mlk, m, n, k, p3, dtype):
     b = randn((m, k), dtype, 1.0, 92)
     bias = randn((1, n), dtype, 1.0, 93)
     a = pack_a(w).cuda()
-    for width in (1, 2, 4):                                   # 128-token panels, 256-token panels, chosen by the library
-        c = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=1, kernelParam2=width, kernelParam3=p3,
+    # (rows, tokens) of a panel: 128 x 128, 256 x 128, 256 x 256, both chosen by the library
+    for rg, width in ((2, 1), (4, 1), (4, 2), (1, 4)):
+        c = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=rg, kernelParam2=width, kernelParam3=p3,
                                     kernelId=3, bias=bias.cuda())
         assert c.shape == (m, n) and c.dtype == dtype
         assert_close(c, ogemm.linear_expected(w, b, 0.5, bias), RTOL, ATOL, "panel n=%d k=%d M=%d" % (n, k, m))
-        c2 = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=1, kernelParam2=width,
+        c2 = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=rg, kernelParam2=width,
                                      kernelParam3=p3, kernelId=3, bias=bias.cuda())
         assert torch.equal(c, c2)
 
@@ -175,9 +176,9 @@ def test_gemm_panel_kernel_soft_fp8(mlk, m, scaled):
     g = torch.Generator().manual_seed(96)
     scale = (torch.rand((n // 128, k // 128), generator=g) * 0.02 + 0.001).float() if scaled else None
     b = randn((m, k), torch.bfloat16, 1.0, 97)
-    for p3, width in ((1, 1), (2, 1), (1, 2), (2, 2)):
+    for p3, rg, width in ((1, 2, 1), (2, 2, 1), (2, 4, 1), (1, 4, 2), (2, 4, 2)):
         c = mlk.gemm_layoutA_soft_fp8_wapper(pack_a(codes).cuda(), None if scale is None else scale.cuda(), b.cuda(),
-                                             n, m, k, kernelParam1=1, kernelParam2=width, kernelParam3=p3, kernelId=3)
+                                             n, m, k, kernelParam1=rg, kernelParam2=width, kernelParam3=p3, kernelId=3)
         want = ogemm.softfp8_linear_expected(codes.numpy(), None if scale is None else scale.numpy(), b)
         assert_close(c, want, RTOL, ATOL, "panel fp8 M=%d slices=%d width=%d" % (m, p3, width))
 

@@ -15,6 +15,7 @@ def test_gemm_guard_accepts_both_kernels_and_rejects_bad_rows():
     assert ops._gemm_guard((4, 1, 2, 1), 11008) == (4, 1, 2, 1)      # one workgroup per CU
     assert ops._gemm_guard((18, 8, 4, 1), 28672) == (18, 8, 4, 1)    # eight row groups per wave
     assert ops._gemm_guard((3, 1, 1, 2), 11008) == (3, 1, 1, 2)      # panel kernel
+    assert ops._gemm_guard((3, 2, 4, 2), 272) == (3, 2, 4, 2)        # its row groups per wave need not divide N/16
     assert ops._gemm_guard((5, 1, 1, 1), 11008) == (1, 1, 4, 1)      # unknown kernel id
     assert ops._gemm_guard((1, 3, 4, 1), 11008) == (1, 1, 4, 1)      # row groups per wave not in {1,2,4}
     assert ops._gemm_guard((1, 4, 4, 1), 16 * 6) == (1, 1, 4, 1)     # 6 row groups are not a multiple of 4
@@ -71,18 +72,19 @@ def test_beta_must_be_zero():
     ops._check_beta(0)
 
 
-def test_panel_kernel_default_and_k_slices():
-    """Unscanned row-major shapes: the panel kernel from about a hundred tokens on, with as many K slices as
-    keep 256-row x 128-token panels x slices within the CU count."""
+def test_panel_kernel_default_shape():
+    """Unscanned row-major shapes: the panel kernel from about a hundred tokens on; 128-row panels while there
+    are few of them, and as many K slices as keep panels x slices within the CU count."""
     from muxi_native_layout_kernels_amd import arg_selector as sel
-    assert sel.panel_k_slices(11008, 128, 4096) == 4          # 43 panels
-    assert sel.panel_k_slices(11008, 256, 4096) == 2          # 86 panels
-    assert sel.panel_k_slices(11008, 512, 4096) == 1          # 172 panels
-    assert sel.panel_k_slices(8192, 256, 8192) == 4           # 64 panels
-    assert sel.panel_k_slices(28672, 128, 8192) == 2          # 112 panels
-    assert sel.panel_k_slices(1024, 128, 1024) == 2           # 8 windows: at least four per slice
-    assert sel.panel_k_slices(1024, 128, 384) == 1
-    assert sel._gemm_default_rowmajor(11008, 512, 4096) == (3, 1, 4, 1)
+    assert sel.panel_shape(11008, 128, 4096) == (2, 2)         # 43 panels of 256 rows -> 86 of 128 rows
+    assert sel.panel_shape(11008, 256, 4096) == (2, 1)         # 86 -> 172
+    assert sel.panel_shape(11008, 512, 4096) == (4, 1)         # 172 panels
+    assert sel.panel_shape(8192, 128, 8192) == (2, 4)          # 32 -> 64
+    assert sel.panel_shape(8192, 512, 8192) == (4, 2)          # 128 panels
+    assert sel.panel_shape(28672, 128, 8192) == (4, 2)         # 112 panels
+    assert sel.panel_shape(1024, 128, 1024) == (2, 2)          # 8 windows: at least four per slice
+    assert sel.panel_shape(1024, 128, 384) == (2, 1)
+    assert sel._gemm_default_rowmajor(11008, 512, 4096) == (3, 4, 4, 1)
     assert sel._gemm_default_rowmajor(11008, 96, 4096)[0] == 2      # still the row-shared kernel
     assert sel._gemm_default_rowmajor(11008, 512, 4096 + 64)[0] == 2  # K is no multiple of 128
     assert sel._gemm_default(11008, 512, 4096)[0] == 2              # native operands never get the panel kernel
