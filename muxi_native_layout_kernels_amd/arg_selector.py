@@ -21,7 +21,7 @@ What the columns select on gfx950 (the rows are produced by the scripts in
                 kernelId     1 = wave-tiled MFMA kernel (waves of a workgroup split K)
                              2 = row-shared tile kernel (4 waves share the activations of
                                  each k window through LDS; kernelParam2 is not used)
-                             3 = panel kernel for more than about a hundred tokens (256 weight
+                             3 = panel kernel for more than 64 tokens (128 or 256 weight
                                  rows x 128 tokens per workgroup, 32x32x16 MFMA, any number of
                                  tokens in one launch; row-major operands, K % 128 == 0;
                                  kernelParam1 = 2: panels of 128 rows, 4: of 256 rows,
@@ -149,9 +149,9 @@ def panel_shape(n, m, k, cus=256):
 
 
 def _gemm_default_rowmajor(n, m, k):
-    """Row-major activations and output: from about a hundred tokens on the product is bound by the matrix
-    cores and the panel kernel (id 3) takes over (panel width left to the library)."""
-    if m > 96 and k % 128 == 0:
+    """Row-major activations and output: above 64 tokens the panel kernel (id 3) takes over (measured ahead of
+    the row-shared kernel from 72 tokens on; panel width left to the library)."""
+    if m > 64 and k % 128 == 0:
         rg, sk = panel_shape(n, m, k)
         return (3, rg, 4, sk)
     return _gemm_default(n, m, k)

@@ -132,7 +132,7 @@ def test_gemm_tile_kernel_wide_passes(mlk, m, p1, p3):
 
 
 def test_gemm_wide_default_parameters(mlk):
-    """A shape that is in no table: above 64 tokens the heuristic picks the row-shared kernel."""
+    """A shape that is in no table, above 64 tokens: the heuristic picks the panel kernel (K % 128 == 0)."""
     n, k, m = 768, 512, 150
     w = randn((n, k), torch.float16, 0.02, 61)
     b = randn((m, k), torch.float16, 1.0, 62)
@@ -184,7 +184,7 @@ def test_gemm_panel_kernel_soft_fp8(mlk, m, scaled):
 
 
 def test_gemm_panel_kernel_is_the_wide_default(mlk):
-    """Above about a hundred tokens the heuristic for unscanned shapes picks the panel kernel; a K that is no
+    """Above 64 tokens the heuristic for unscanned shapes picks the panel kernel; a K that is no
     multiple of 128 keeps the row-shared kernel, and the panel kernel refuses it when asked for by id."""
     from muxi_native_layout_kernels_amd import arg_selector
     assert arg_selector.selector("layoutA_gemm").get_args((4096, 300, 1024))[0] == 3

@@ -73,7 +73,7 @@ def test_beta_must_be_zero():
 
 
 def test_panel_kernel_default_shape():
-    """Unscanned row-major shapes: the panel kernel from about a hundred tokens on; 128-row panels while there
+    """Unscanned row-major shapes: the panel kernel above 64 tokens; 128-row panels while there
     are few of them, and as many K slices as keep panels x slices within the CU count."""
     from muxi_native_layout_kernels_amd import arg_selector as sel
     assert sel.panel_shape(11008, 128, 4096) == (2, 2)         # 43 panels of 256 rows -> 86 of 128 rows
@@ -85,6 +85,7 @@ def test_panel_kernel_default_shape():
     assert sel.panel_shape(1024, 128, 1024) == (2, 2)          # 8 windows: at least four per slice
     assert sel.panel_shape(1024, 128, 384) == (2, 1)
     assert sel._gemm_default_rowmajor(11008, 512, 4096) == (3, 4, 4, 1)
-    assert sel._gemm_default_rowmajor(11008, 96, 4096)[0] == 2      # still the row-shared kernel
+    assert sel._gemm_default_rowmajor(11008, 72, 4096) == (3, 2, 4, 2)
+    assert sel._gemm_default_rowmajor(11008, 64, 4096)[0] == 1      # the narrow kernels up to 64 tokens
     assert sel._gemm_default_rowmajor(11008, 512, 4096 + 64)[0] == 2  # K is no multiple of 128
     assert sel._gemm_default(11008, 512, 4096)[0] == 2              # native operands never get the panel kernel
