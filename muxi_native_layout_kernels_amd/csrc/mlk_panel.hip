@@ -4,7 +4,10 @@
 // A workgroup of four waves computes a panel of 256 weight rows x 128 tokens over one of SK slices
 // of K with v_mfma_f32_32x32x16 (one wave per SIMD issues the 16x16x32 form at little more than half
 // rate; the 32x32 form runs at nine tenths of peak from a single wave).  Every wave owns four row
-// groups (two pairs of 32 rows) and all four blocks of 32 tokens: eight 32x32 accumulators.
+// groups (two pairs of 32 rows) and all four blocks of 32 tokens: eight 32x32 accumulators.  Two other
+// shapes exist: 256 rows x 256 tokens (sixteen accumulators, k windows of 64 instead of 128) when that
+// makes fewer rounds of one workgroup per CU, and 128 rows x 128 tokens (one pair of row groups per
+// wave) while panels are too few to give every CU one.
 //
 // Weights come straight from global memory, two k windows ahead in a register ring.  A layout-A
 // tile (16 rows x 32 k: lane 16 q + r holds row r, k octet q) is not the 32x32x16 operand (lane
@@ -13,10 +16,12 @@
 // 16-lane rows [X0 X1 X2 X3], [Y0 Y1 Y2 Y3] into [X0 Y0 X2 Y2], [X1 Y1 X3 Y3], v_permlane32_swap
 // then into [X0 Y0 X1 Y1] (k octets 0, 1 of rows 0..31) and [X2 Y2 X3 Y3] (octets 2, 3).
 //
-// The activations of a k window (two k tiles, 128 tokens: 16 KiB) are fetched once per workgroup
-// with 16-byte loads one window ahead and parked in LDS in operand order: granule
-// ((w*4 + tb)*4 + octet)*33 + token (+ 4 w), so that an operand is two runs of 32 consecutive
-// granules for ds_read_b128 and the eight granules a token row contributes fall into different banks.
+// The activations of a k window are fetched once per workgroup with 16-byte loads two windows ahead
+// (they wait in registers) and parked in LDS one window ahead in operand order: granule
+// ((t*TB + tb)*4 + octet)*33 + token (+ 4 t) for k tile t, token block tb, so that an operand is two
+// runs of 32 consecutive granules for ds_read_b128 and the granules a token row contributes fall into
+// different banks.  Three LDS buffers, one barrier per window; within a window the LDS reads and the
+// global loads are scheduled between the MFMAs (sched_group_barrier).
 //
 // Grid: the token tiles of one row tile run next to each other on one XCD (workgroup id modulo 8
 // picks the XCD), so the weights of a row tile are read from HBM once and served to the other token
@@ -42,7 +47,7 @@ struct PanelArgs {
     uint16_t *C;
     const uint16_t *bias;
     const float *scale;
-    f32x4 *partial;      // [SK][tiles][4 waves][32][64]
+    f32x4 *partial;      // [SK][tiles][4 waves][quads of a wave][two planes of 64 x 8 bytes]
     int *counters;       // [tiles], zero between calls
     int M, N, K;
     int SK;
