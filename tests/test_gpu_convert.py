@@ -79,3 +79,27 @@ def test_converted_projection_feeds_linear(mlk, tmp_path):
     y = mlk.gemm_layoutA_linear(ck.tensor("proj.weight"), x.cuda(), bias=ck.tensor("proj.bias").view(1, -1))
     want = x.double().numpy() @ w.double().numpy().T + ck.tensor("proj.bias").double().cpu().numpy()
     assert_close(y, want, 1e-2, 1e-2, "linear on a converted projection")
+
+
+def test_cli_converts_a_sharded_checkpoint(mlk, tmp_path, capsys):
+    """The command line end to end: two input shards, the deepseek preset, device packing, the result re-opened."""
+    from muxi_native_layout_kernels_amd import convert as cv
+    E, H, I = 2, 256, 128
+    shard_a, shard_b = {}, {}
+    for e in range(E):
+        for i, (proj, shape) in enumerate((("gate_proj", (I, H)), ("up_proj", (I, H)), ("down_proj", (H, I)))):
+            base = "model.layers.1.mlp.experts.%d.%s" % (e, proj)
+            (shard_a if e == 0 else shard_b)[base + ".weight"] = randn(shape, torch.bfloat16, 0.02, 10 * e + i)
+    shard_b["model.layers.1.mlp.gate.weight"] = randn((E, H), torch.bfloat16, 0.1, 77)
+    pa, pb, dst = str(tmp_path / "a.safetensors"), str(tmp_path / "b.safetensors"), str(tmp_path / "out.safetensors")
+    save_file(shard_a, pa)
+    save_file(shard_b, pb)
+    cv.main(["--preset", "deepseek", pa, pb, dst])
+    assert "wrote" in capsys.readouterr().out
+    ck = cv.PackedCheckpoint(dst)
+    w1 = ck.tensor("model.layers.1.mlp.experts.w1")
+    assert tuple(w1.shape) == (E, 2 * I // 16, H // 8, 16, 8)
+    gate1 = shard_b["model.layers.1.mlp.experts.1.gate_proj.weight"]
+    up1 = shard_b["model.layers.1.mlp.experts.1.up_proj.weight"]
+    assert torch.equal(w1[1].cpu(), pack_a(torch.cat([gate1, up1], 0)))
+    assert ck.info("model.layers.1.mlp.gate.weight")["layout"] == "plain"
