@@ -43,6 +43,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--quick", action="store_true", help="headline workload only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--case", default=None,
+                    help="besides the headline, run only the per-configuration cases whose name contains this text "
+                         "(for profiling one kernel)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain copy kernel of known size (256 MiB in, 256 MiB out) so that "
                          "hardware byte counters can be scaled against it")
@@ -288,6 +291,11 @@ def main():
     N, K_, M = 11008, 4096, 16
     head = gemm_case("C2 fp16 gemm_layoutA 11008x4096 M=16", N, K_, 0, M, args.steps, args.warmup)
     per_config = []
+
+    def add(case, name, *a, **kw):
+        """Run one per-configuration case unless --case asks for others only."""
+        if args.case is None or args.case in name:
+            per_config.append(case(name, *a, **kw))
     ceiling = None
     resident = None
     if not args.quick:
@@ -302,29 +310,29 @@ def main():
         same_size = wbytes / read_ceiling(min(args.steps, 100), wbytes - wbytes % 4096, copies_for(wbytes),
                                           ((512, 1024), (1024, 512), (256, 2048), (512, 512))) / 1e3
         short = max(20, min(args.steps, 100))
-        per_config.append(gemv_case("C1 bf16 gemv 4096x4096", 4096, 4096, 1, short, 10))
+        add(gemv_case, "C1 bf16 gemv 4096x4096", 4096, 4096, 1, short, 10)
         for m in (1, 8, 32, 64):
-            per_config.append(gemm_case("C2 fp16 gemm_layoutA 11008x4096 M=%d" % m, N, K_, 0, m, short, 10))
-        per_config.append(gemv_case("C2 fp16 gemv 11008x4096", N, K_, 0, short, 10))
-        per_config.append(gemv_case("C3 soft-fp8 gemv 28672x8192", 28672, 8192, 2, short, 10))
+            add(gemm_case, "C2 fp16 gemm_layoutA 11008x4096 M=%d" % m, N, K_, 0, m, short, 10)
+        add(gemv_case, "C2 fp16 gemv 11008x4096", N, K_, 0, short, 10)
+        add(gemv_case, "C3 soft-fp8 gemv 28672x8192", 28672, 8192, 2, short, 10)
         for m in (4, 16):
-            per_config.append(gemm_case("C3 soft-fp8 gemm_layoutA 28672x8192 M=%d" % m, 28672, 8192, 2, m, short, 10))
-        per_config.append(gemm_case("C4 bf16 gemm_layoutABC+reLayoutC 8192x8192 M=32", 8192, 8192, 1, 32, short, 10,
-                                    native=True))
+            add(gemm_case, "C3 soft-fp8 gemm_layoutA 28672x8192 M=%d" % m, 28672, 8192, 2, m, short, 10)
+        add(gemm_case, "C4 bf16 gemm_layoutABC+reLayoutC 8192x8192 M=32", 8192, 8192, 1, 32, short, 10,
+                                    native=True)
         for T in (1, 16, 64, 256):
-            per_config.append(moe_case("C5 bf16 fused_moe T=%d" % T, T, False, 20, 5))
+            add(moe_case, "C5 bf16 fused_moe T=%d" % T, T, False, 20, 5)
         for T in (1, 16):
-            per_config.append(moe_case("C5 soft-fp8 fused_moe T=%d" % T, T, True, 20, 5))
+            add(moe_case, "C5 soft-fp8 fused_moe T=%d" % T, T, True, 20, 5)
         for T in (1, 16):
-            per_config.append(moe_next_case("next: grouped-routing MoE E=256 top-8 H=7168 I=2048 bf16 T=%d" % T, T, 20, 5))
+            add(moe_next_case, "next: grouped-routing MoE E=256 top-8 H=7168 I=2048 bf16 T=%d" % T, T, 20, 5)
         moe_w.clear()
         torch.cuda.empty_cache()
         for m in (128, 256, 1024, 4096):
-            per_config.append(panel_case("next: prefill gemm_layoutA fp16 11008x4096 M=%d" % m, N, K_, 0, m, 20))
-        per_config.append(panel_case("next: prefill gemm_layoutA bf16 8192x8192 M=4096", 8192, 8192, 1, 4096, 10))
-        per_config.append(panel_case("next: prefill gemm_layoutA soft-fp8 28672x8192 M=1024", 28672, 8192, 2, 1024, 10))
+            add(panel_case, "next: prefill gemm_layoutA fp16 11008x4096 M=%d" % m, N, K_, 0, m, 20)
+        add(panel_case, "next: prefill gemm_layoutA bf16 8192x8192 M=4096", 8192, 8192, 1, 4096, 10)
+        add(panel_case, "next: prefill gemm_layoutA soft-fp8 28672x8192 M=1024", 28672, 8192, 2, 1024, 10)
         torch.cuda.empty_cache()
-        per_config.append(pack_case("next: checkpoint conversion, pack_layout_a bf16 [8, 28672, 4096]", 8, 28672, 4096, 10))
+        add(pack_case, "next: checkpoint conversion, pack_layout_a bf16 [8, 28672, 4096]", 8, 28672, 4096, 10)
         torch.cuda.empty_cache()
         for row in per_config:
             row.pop("wall", None)
