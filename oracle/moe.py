@@ -49,7 +49,7 @@ def torch_path_fused_moe(hidden, w1, w2, gating, topk, num_expert_group=1, topk_
         gsc = grouped.max(dim=-1).values                           # utils.py:180-181
     gidx = torch.topk(gsc, k=topk_group, dim=-1, sorted=False)[1]  # utils.py:185-186
     gmask = torch.zeros_like(gsc).scatter_(1, gidx, 1)
-    emask = gmask.unsqueeze(-1).expand(n_tok, num_expert_group, n_exp // num_expert_group)
+    emask = gmask.unsqueeze(-1).expand(n_tok, num_expert_group, sc.shape[-1] // num_expert_group)  # utils.py:189-191
     masked = sc.masked_fill(~emask.reshape(n_tok, -1).bool(), 0.0)  # utils.py:192-196
     if bias is not None:
         ids = torch.topk(masked, k=topk, dim=-1, sorted=False)[1]  # utils.py:199

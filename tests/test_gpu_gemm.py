@@ -282,6 +282,8 @@ def test_native_chain_config(mlk):
     c_nat = mlk.gemm_layoutABC(a, b_nat)
     c = mlk.reLayoutC(c_nat)
     assert_close(c, ogemm.linear_expected(w, b), RTOL, ATOL, "ABC 8192")
+    # the native output is layout-C of the row-major one (oracle permutation, bit for bit)
+    assert torch.equal(c_nat.cpu(), ogemm.layout_c_of(c.cpu()))
     # chain a second product on the native output: C1 is the layout-B operand of the next layer
     w2 = randn((256, n), torch.bfloat16, 0.02, 2027)
     c2 = mlk.reLayoutC(mlk.gemm_layoutABC(pack_a(w2).cuda(), c_nat))

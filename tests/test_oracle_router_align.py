@@ -87,6 +87,36 @@ def test_router_grouped_with_bias_brute_force():
         assert torch.equal(w[t], p[t][ids[t].long()])
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("score_fun", [0, 1])
+@pytest.mark.parametrize("E,n_groups,topk_groups,K", [(32, 8, 4, 8), (256, 8, 4, 8), (64, 4, 2, 6), (48, 6, 1, 3)])
+def test_router_grouped_without_bias_brute_force(dtype, score_fun, E, n_groups, topk_groups, K):
+    """No bias: the group score is the largest score of the group (fused_topK.h:136-171).  Independent
+    ranking: groups by (-max, group id), then the experts of the kept groups by (-score, id)."""
+    T = 48
+    logits = randn((T, E), dtype, 1.5, 100 + E)
+    ids, w = router.route(logits, score_fun, n_groups, topk_groups, K)
+    p = router.scores(logits, score_fun).double().numpy()
+    per = E // n_groups
+    for t in range(T):
+        gmax = [p[t, g * per:(g + 1) * per].max() for g in range(n_groups)]
+        kept = sorted(range(n_groups), key=lambda g: (-gmax[g], g))[:topk_groups]
+        cand = [j for j in range(E) if j // per in kept]
+        want = sorted(cand, key=lambda j: (-p[t, j], j))[:K]
+        got = ids[t].tolist()
+        assert (sorted(want) == got) if score_fun == 0 else (want == got)
+        assert all(g // per in kept for g in got)
+        for k in range(K):
+            assert w[t, k].double().item() == p[t, got[k]]
+
+
+def test_router_grouped_one_group_equals_plain():
+    logits = randn((32, 64), torch.bfloat16, 1.0, 8)
+    a = router.route(logits, 1, 1, 1, 6)
+    b = router.route(logits, 1, 8, 8, 6)          # every group kept: the mask removes nothing
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
 def test_renormalize():
     w = torch.tensor([[0.25, 0.5], [0.125, 0.125]], dtype=torch.bfloat16)
     r = router.renormalize(w)

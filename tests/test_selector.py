@@ -21,14 +21,46 @@ def test_excerpt_known_answers_oracle_and_product_agree():
     assert got[(19008, 5120)] == (256, 1, 1, 8)
 
 
-def test_known_answer_rows_parse():
-    rows = [l for l in open(os.path.join(GOLD, "selector_rows.csv")).read().splitlines() if not l.startswith("#")]
-    for line in rows:
+def _golden_rows():
+    """(table file, line number in the reference's table, cells) of every known-answer row."""
+    out = []
+    for line in open(os.path.join(GOLD, "selector_rows.csv")).read().splitlines():
+        if line.startswith("#"):
+            continue
         fname, lineno, row = line.split(",", 2)
-        cells = [int(c) for c in row.strip('"').split(",")]
-        nkey = 2 if "gemv" in fname else 3
-        table = osel.parse_table("header\n" + ",".join(map(str, cells)), nkey)
-        assert table[tuple(cells[:nkey])] == tuple(cells[nkey:])
+        out.append((fname, int(lineno), [int(c) for c in row.strip('"').split(",")]))
+    return out
+
+
+def test_known_answer_rows_through_a_multi_row_table(tmp_path):
+    """The reference-held rows are looked up through whole tables built around them: a header, decoy rows
+    with other keys before and after, an earlier duplicate of the key with other values (the later row
+    must win) and a row with too few cells (skipped).  Oracle and product must both return the
+    reference's answer."""
+    for nkey, fallback in ((2, arg_selector.GEMV_FALLBACK), (3, arg_selector.GEMM_FALLBACK)):
+        rows = [cells for fname, _, cells in _golden_rows() if len(cells) == nkey + 4]
+        assert rows
+        lines = ["header"]
+        for i, cells in enumerate(rows):
+            key, val = cells[:nkey], cells[nkey:]
+            decoy_key = [key[0] + 16 * (i + 1)] + key[1:]
+            lines.append(",".join(map(str, decoy_key + [7, 7, 7, 7])))
+            lines.append(",".join(map(str, key + [v + 1 for v in val])))          # earlier duplicate, loses
+            lines.append(",".join(map(str, key[:nkey] + val[:2])))                 # wrong cell count, skipped
+            lines.append(",".join(map(str, cells)))                                # the reference's row, wins
+            lines.append(",".join(map(str, [key[0] + 32 * (i + 1)] + key[1:] + [9, 9, 9, 9])))
+        text = "\n".join(lines) + "\n"
+        want_table = osel.parse_table(text, nkey)
+        path = tmp_path / ("table%d.csv" % nkey)
+        path.write_text(text)
+        sel = arg_selector._Selector(str(path), nkey, fallback, "golden")
+        sel.path = lambda path=path: str(path)
+        for cells in rows:
+            key, val = tuple(cells[:nkey]), tuple(cells[nkey:])
+            assert osel.lookup(want_table, key, fallback) == val
+            assert sel.get_args(key) == val
+        miss = tuple([5] * nkey)
+        assert osel.lookup(want_table, miss, fallback) == fallback
 
 
 def test_fallbacks_and_guards_oracle():
