@@ -6,8 +6,14 @@
  * is cited beside it.  All pointers are DEVICE pointers unless said otherwise,
  * all matrices are dense and contiguous, and every call only enqueues work on
  * `stream` (a hipStream_t passed as void*; NULL = the default stream): nothing
- * is allocated, nothing is synchronised, no global state is kept besides the
- * last error text of the calling thread.
+ * is allocated and nothing is synchronised.
+ *
+ * State the library keeps for the whole process: the last error text (per
+ * calling thread); the experiment switches of mlk_set_tunable() and
+ * mlk_moe_set_tile_path() (plain ints, not thread-safe: set them before other
+ * threads call in, they change what every later call launches); per device,
+ * the compute-unit count and which kernels have had their LDS limit raised
+ * (both written once, safe to race).
  *
  * Naming follows the reference: weights are "A" [N rows = output features,
  * K reduction], activations are "B" [M tokens, K], outputs are "C" [M, N].
@@ -223,6 +229,14 @@ int mlk_fused_experts_compute(const void *w1, const void *w2, const void *x, int
                               const float *w2_scale, void *y, void *workspace, size_t workspace_bytes,
                               void *stream);
 size_t mlk_moe_workspace_bytes(int n_tokens, int n_experts, int topk, int hidden, int inter);
+
+/* How mlk_fused_experts_compute would run one pass of min(n_tokens, 256) tokens, decided on the host from the
+ * sizes alone (no GPU is touched): out[0] = kernel family (0 single-token GeMV kernels, 1 decode kernels that
+ * align in-kernel, 2 decode kernels after the alignment kernel, 3 row-shared kernels), out[1] = token blocks
+ * per task, out[2] = upper bound of the task list, out[3] = row groups per wave and out[4] = K slices of the
+ * down projection, out[5] = waves and out[6] = dynamic LDS bytes of the decode down kernel (families 1, 2),
+ * out[7] = its static LDS bytes.  For tests and the tuning scripts; no counterpart in the reference. */
+int mlk_moe_plan(int n_tokens, int n_experts, int topk, int hidden, int inter, int w_kind, int32_t *out);
 
 #ifdef __cplusplus
 }

@@ -40,6 +40,7 @@ SIGNATURES = {
                                           c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                           c_void_p, c_size_t, c_void_p]),
     "mlk_moe_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
+    "mlk_moe_plan": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
 }
 
 _lock = threading.Lock()

@@ -28,6 +28,9 @@ extern int g_tunable[8];
 // Record an error message for mlk_last_error() and return the code.
 int fail(int code, const char *msg);
 
+// Compute units of the current device (cached per device; 256 if the runtime cannot tell).
+int device_cus();
+
 #define MLK_REQUIRE(cond, msg)                                                  \
     do {                                                                        \
         if (!(cond)) return ::mlk::fail(MLK_ERR_INVALID, msg);                  \

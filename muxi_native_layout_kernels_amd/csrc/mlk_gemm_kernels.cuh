@@ -520,13 +520,7 @@ static int launch_balanced(const GemmArgs &p, int wgs, hipStream_t s) {
 
 // number of workgroups for kernel id 4 and the larger of the two row-group counts, or 0 when it does not apply
 static int balanced_grid(const GemmArgs &p, int CB, int *r_max) {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) != hipSuccess || hipGetDeviceProperties(&prop, dev) != hipSuccess) return 0;
-        cus = prop.multiProcessorCount;
-    }
+    const int cus = device_cus();
     const int groups = p.N / 16;
     if (groups <= cus) return 0;
     const int r = (groups + cus - 1) / cus;

@@ -1166,16 +1166,42 @@ static size_t carve(uint8_t *base, int tc, int E, int K, int hidden, int inter, 
     return off;
 }
 
+// Waves and dynamic LDS of the decode down kernel for R row groups per wave and CB token blocks per task:
+// [WK][R*CB] accumulator tiles for the wave fold plus the fp32 output tile [T][16 R], next to the kernel's
+// static tables, inside the 64 KiB a workgroup gets without a per-kernel attribute.  False when even a single
+// wave does not fit (R = 4 with more than 224 tokens).
+static bool moe_down_shape(int T, int R, int CB, int *wk, size_t *lds) {
+    auto need = [&](int w) { return (size_t)w * R * CB * 1024 + (size_t)T * 16 * R * 4; };
+    const size_t budget = 64 * 1024 - sizeof(DecodeTables) - 64;
+    int w = 16;
+    while (w > 1 && (w * 64 > max_threads_for_tiles(R * CB) || need(w) > budget)) w >>= 1;
+    *wk = w;
+    *lds = need(w);
+    return need(w) <= budget;
+}
+
+// Row groups per wave (= K slices across workgroups) of the decode down kernel with one token block per
+// task.  More row groups cut the re-reads of the intermediate, but the output tile grows with them: the
+// preferred count is halved until the tile fits with at least four waves left to stream weights.
+static int moe_down_rows(int T, int H, int I, bool fp8) {
+    int r = g_tunable[7] ? g_tunable[7] : (fp8 ? 4 : 1);
+    if (r != 1 && r != 2 && r != 4) r = 1;
+    for (; r > 1; r >>= 1) {
+        int wk;
+        size_t lds;
+        if ((H / 16) % r == 0 && (I / 32) % r == 0 && moe_down_shape(T, r, 1, &wk, &lds) && wk >= 4) break;
+    }
+    return r;
+}
+
 template <class T, bool FP8, int CB, int R, bool INLINE>
 static int launch_moe_down(const MoeArgs &a, int skd, hipStream_t s) {
     constexpr int U2F = (R * CB >= 4) ? 4 : (R * CB == 1 ? 10 : 6);   // fp8 tiles are half as many bytes
     constexpr int U2 = FP8 && CB == 1 ? U2F : ((R * CB >= 4) ? 3 : (R * CB == 1 ? 8 : 4));
     MoeArgs d = a;
-    d.WK = 16;
-    while (d.WK > 1 && (d.WK * 64 > max_threads_for_tiles(R * CB) ||
-                        (size_t)d.WK * R * CB * 1024 + (size_t)a.T * 16 * R * 4 + sizeof(DecodeTables) > 64 * 1024))
-        d.WK >>= 1;
-    size_t lds2 = (size_t)d.WK * R * CB * 1024 + (size_t)a.T * 16 * R * 4;
+    size_t lds2;
+    if (!moe_down_shape(a.T, R, CB, &d.WK, &lds2))
+        return fail(MLK_ERR_INVALID, "moe: the down projection's output tile does not fit the workgroup's LDS");
     moe_down_kernel<T, FP8, CB, R, U2, INLINE><<<dim3(a.H / 16 / R, skd), d.WK * 64, lds2, s>>>(d);
     MLK_LAUNCH_CHECK();
     return MLK_OK;
@@ -1198,15 +1224,29 @@ static int launch_moe(const MoeArgs &a, int max_tasks, hipStream_t s) {
     if constexpr (CB == 1) {
         // One token block: R row groups per wave cut the re-reads of the intermediate R-fold; K is
         // sliced R ways so that the grid still has a workgroup per 16 output rows.
-        const int r = g_tunable[7] ? g_tunable[7] : (FP8 ? 4 : 1);
-        const int tiles = a.I / 32;
-        if (r == 2 && (a.H / 16) % 2 == 0 && tiles % 2 == 0) return launch_moe_down<T, FP8, CB, 2, INLINE>(a, 2, s);
-        if (r == 4 && (a.H / 16) % 4 == 0 && tiles % 4 == 0) return launch_moe_down<T, FP8, CB, 4, INLINE>(a, 4, s);
+        const int r = moe_down_rows(a.T, a.H, a.I, FP8);
+        if (r == 2) return launch_moe_down<T, FP8, CB, 2, INLINE>(a, 2, s);
+        if (r == 4) return launch_moe_down<T, FP8, CB, 4, INLINE>(a, 4, s);
     }
     return launch_moe_down<T, FP8, CB, 1, INLINE>(a, 1, s);
 }
 
 constexpr int kMoeMaxKSlices = 8;  // K slices of the row-shared down projection (sizes its fp32 buffer)
+
+// Row groups per wave and K slices of the row-shared down projection for CB token blocks per task.
+static int moe_tile_down_rows(int cb, int H) {
+    const int r = cb > 4 ? 4 : 2;
+    return (H / 16) % (r * kTileWaves) == 0 ? r : 1;
+}
+static int moe_tile_down_slices(int cb, int H, int I, int max_tasks) {
+    const int r = moe_tile_down_rows(cb, H);
+    if (r == 1) return 1;
+    const int row_tiles = (H / 16) / (r * kTileWaves);
+    const int windows = (I / 32) / (cb > 4 ? 2 : 4);
+    int skd = 1;
+    while (skd < kMoeMaxKSlices && row_tiles * max_tasks * skd < 512 && windows % (skd * 2) == 0) skd *= 2;
+    return skd;
+}
 
 template <class T, bool FP8, int CB>
 static int launch_moe_tile(const MoeArgs &a, int max_tasks, float *obuf, hipStream_t s) {
@@ -1219,11 +1259,9 @@ static int launch_moe_tile(const MoeArgs &a, int max_tasks, float *obuf, hipStre
     // workgroups by slicing K, each slice a whole number of windows
     constexpr int R = CB > 4 ? 4 : 2;
     const int groups_h = a.H / 16;
-    const int windows = (a.I / 32) / tile_kw<CB>();
     if (groups_h % (R * kTileWaves) == 0) {
         const int row_tiles = groups_h / (R * kTileWaves);
-        int skd = 1;
-        while (skd < kMoeMaxKSlices && row_tiles * max_tasks * skd < 512 && windows % (skd * 2) == 0) skd *= 2;
+        const int skd = moe_tile_down_slices(CB, a.H, a.I, max_tasks);
         moe_down_tile_kernel<T, FP8, CB, R><<<dim3(row_tiles, max_tasks, skd), 256, tile_lds_bytes<CB>(), s>>>(a, obuf);
         MLK_LAUNCH_CHECK();
         moe_combine_kernel<T><<<dim3(a.T, (a.H + 1023) / 1024), 256, 0, s>>>(obuf, a.Y, a.topk_ids, a.experts_map, a.K, a.H, a.E, skd);
@@ -1250,9 +1288,65 @@ static int launch_moe_cb(const MoeArgs &a, int cb, int max_tasks, bool inline_al
     }
 }
 
+// How one pass of up to kMoeChunk tokens is run.  The launch code below and mlk_moe_plan() both read it.
+enum { kMoePathGemv1 = 0, kMoePathDecodeInline = 1, kMoePathDecode = 2, kMoePathTile = 3 };
+struct MoePlan {
+    int path;         // kMoePath*
+    int cb;           // token blocks per task
+    int max_tasks;    // upper bound of the task list (grid dimension)
+    int down_r;       // down projection: row groups per wave
+    int down_slices;  // down projection: K slices across workgroups
+    int down_wk;      // decode down kernel: waves per workgroup
+    size_t down_lds;  // decode down kernel: dynamic LDS bytes
+};
+static MoePlan moe_plan(int tc, int n_experts, int topk, int hidden, int inter, bool fp8) {
+    MoePlan pl = {};
+    const int n_pairs = tc * topk;
+    pl.cb = moe_blocks_per_task(tc, topk, n_experts);
+    const int active = n_experts < n_pairs ? n_experts : n_pairs;
+    pl.max_tasks = active + n_pairs / (16 * pl.cb);
+    pl.down_r = pl.down_slices = 1;
+    if (g_moe_gemv1 && tc == 1 && topk <= 16 && (size_t)topk * inter * 2 <= 56 * 1024 &&
+        (size_t)hidden * 2 <= 56 * 1024 && (!fp8 || (hidden % 64 == 0 && inter % 64 == 0))) {
+        pl.path = kMoePathGemv1;
+        return pl;
+    }
+    const bool inline_align = tc <= 16 && n_pairs <= kDecodePairs;
+    if (inline_align) pl.cb = 1;
+    if (!inline_align && pl.cb >= 2 && (moe_tile_path() || pl.cb > 4)) {
+        pl.path = kMoePathTile;
+        pl.down_r = moe_tile_down_rows(pl.cb, hidden);
+        pl.down_slices = moe_tile_down_slices(pl.cb, hidden, inter, pl.max_tasks);
+        return pl;
+    }
+    pl.path = inline_align ? kMoePathDecodeInline : kMoePathDecode;
+    if (pl.cb == 1) pl.down_r = pl.down_slices = moe_down_rows(tc, hidden, inter, fp8);
+    moe_down_shape(tc, pl.down_r, pl.cb, &pl.down_wk, &pl.down_lds);
+    return pl;
+}
+
 }  // namespace mlk
 
 using namespace mlk;
+
+extern "C" int mlk_moe_plan(int n_tokens, int n_experts, int topk, int hidden, int inter, int w_kind, int32_t *out) {
+    MLK_REQUIRE(out != nullptr, "moe plan: null pointer");
+    MLK_REQUIRE(n_tokens >= 1 && n_experts >= 1 && n_experts <= kMaxExperts && topk >= 1 && topk <= kMaxTopK,
+                "moe plan: sizes out of range");
+    MLK_REQUIRE(hidden > 0 && inter > 0 && hidden % 128 == 0 && inter % 128 == 0,
+                "moe: hidden and intermediate sizes must be multiples of 128");
+    const int tc = n_tokens < kMoeChunk ? n_tokens : kMoeChunk;
+    const MoePlan pl = moe_plan(tc, n_experts, topk, hidden, inter, w_kind == MLK_FP8_E4M3);
+    out[0] = pl.path;
+    out[1] = pl.cb;
+    out[2] = pl.max_tasks;
+    out[3] = pl.down_r;
+    out[4] = pl.down_slices;
+    out[5] = pl.down_wk;
+    out[6] = (int32_t)pl.down_lds;
+    out[7] = (int32_t)sizeof(DecodeTables);
+    return MLK_OK;
+}
 
 extern "C" void mlk_moe_set_tile_path(int on) {
     g_moe_tile = on & 1;
@@ -1329,17 +1423,16 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
     for (int t0 = 0; t0 < n_tokens; t0 += kMoeChunk) {
         const int tc = n_tokens - t0 < kMoeChunk ? n_tokens - t0 : kMoeChunk;
         const int n_pairs = tc * topk;
+        const MoePlan pl = moe_plan(tc, n_experts, topk, hidden, inter, fp8);
         const int cb = moe_blocks_per_task(tc, topk, n_experts);
         MoeWorkspace ws;
         carve((uint8_t *)workspace, tc, n_experts, topk, hidden, inter, &ws);
         const int max_padded = n_pairs + n_experts * 15;
         int max_blocks = (max_padded + 15) / 16;
         if (max_blocks < kDecodePairs) max_blocks = kDecodePairs;
-        const int active = n_experts < n_pairs ? n_experts : n_pairs;
-        const int max_tasks = active + n_pairs / (16 * cb);
+        const int max_tasks = pl.max_tasks;
         // one token: every routed pair is a GeMV with the activations in LDS
-        if (g_moe_gemv1 && tc == 1 && topk <= 16 && (size_t)topk * inter * 2 <= 56 * 1024 &&
-            (size_t)hidden * 2 <= 56 * 1024 && (!fp8 || (hidden % 64 == 0 && inter % 64 == 0))) {
+        if (pl.path == kMoePathGemv1) {
             Moe1Args m;
             m.W1 = (const uint8_t *)w1;
             m.W2 = (const uint8_t *)w2;
@@ -1389,7 +1482,7 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
             continue;
         }
         // decode-sized batches align inside the GeMM kernels; larger ones run the alignment kernel
-        const bool inline_align = tc <= 16 && n_pairs <= kDecodePairs;
+        const bool inline_align = pl.path == kMoePathDecodeInline;
         if (!inline_align) {
             moe_align_kernel<<<1, 1024, 0, s>>>(topk_ids + (size_t)t0 * topk, n_pairs, n_experts, experts_map,
                                                 ws.sorted, ws.cumsum, ws.padded, ws.experts_ids, max_blocks, ws.tasks,

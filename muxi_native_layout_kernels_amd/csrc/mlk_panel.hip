@@ -344,13 +344,7 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
 // Tokens per panel when the caller leaves the choice open.  Workgroups run one per CU in rounds, and a 256-token
 // panel takes 1.84 times as long as a 128-token one (measured), so the width with the cheaper sum of rounds wins.
 int panel_tokens(int m, int n) {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0;
-        hipDeviceProp_t prop;
-        if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) cus = prop.multiProcessorCount;
-        if (cus <= 0) cus = 256;
-    }
+    const int cus = device_cus();
     const long long row_tiles = (n + kPanelRowsPerWg - 1) / kPanelRowsPerWg;
     const long long rounds128 = (row_tiles * ((m + 127) / 128) + cus - 1) / cus;
     const long long rounds256 = (row_tiles * ((m + 255) / 256) + cus - 1) / cus;
@@ -393,9 +387,7 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
     if (hipGetDevice(&dev) != hipSuccess) dev = 0;
     if (width == 256) rows = 256;
     if (rows != 128 && rows != 256) {
-        int cus = 256;
-        hipDeviceProp_t prop;
-        if (hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0) cus = prop.multiProcessorCount;
+        const int cus = device_cus();
         // few panels: 128-row panels put twice as many CUs to work (a 128-row panel takes two thirds of the time of
         // a 256-row one); from three eighths of the CU count on, 256-row panels and K slices fill the chip better
         const long long panels256 = (long long)((n + 255) / 256) * p.token_tiles;

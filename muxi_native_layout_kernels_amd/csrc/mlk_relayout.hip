@@ -1,6 +1,8 @@
 // Relayout kernels: layout-A pack / unpack, layout-B pack, layout-C unpack and
 // the fp8 byte repack.  All are pure permutations, one 16-byte (or 8-byte)
 // granule per thread, writes coalesced; HBM-bound copies.
+#include <atomic>
+
 #include "mlk_common.cuh"
 
 namespace mlk {
@@ -13,6 +15,20 @@ int fail(int code, const char *msg) {
     for (; msg[i] && i < 255; ++i) g_err[i] = msg[i];
     g_err[i] = 0;
     return code;
+}
+
+int device_cus() {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 256;
+    if (dev >= 0 && dev < 64) {
+        const int hit = cached[dev].load(std::memory_order_relaxed);
+        if (hit > 0) return hit;
+    }
+    int cus = 0;
+    if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+    if (dev >= 0 && dev < 64) cached[dev].store(cus, std::memory_order_relaxed);
+    return cus;
 }
 
 // One granule of 8 elements: G = uint4 for 16-bit elements, uint2 for bytes.

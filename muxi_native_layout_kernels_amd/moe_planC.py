@@ -5,7 +5,8 @@ Three library calls per layer: router (scores, grouped selection, top-K and the
 optional renormalisation in one kernel), then alignment + grouped gate/up GeMM +
 grouped down GeMM inside `mlk_fused_experts_compute`.  Apart from the output
 nothing is allocated after the first call of a given shape: routing tables and
-the kernel workspace are cached per device.
+the kernel workspace are cached per device and stream and are never freed, so a
+HIP graph captured around this function stays valid whatever runs later.
 """
 import threading
 from typing import List, Optional
@@ -18,13 +19,15 @@ _cache_lock = threading.Lock()
 _route_cache = {}
 
 
-def _routing_buffers(n_tokens, topk, dtype, device):
-    key = (n_tokens, topk, dtype, device.type, device.index)
+def _routing_buffers(n_tokens, topk, dtype, device, stream=None):
+    """Routing tables (ids, weights) per shape, device and stream.  Entries are never dropped: the kernels get
+    raw pointers, and a HIP graph captured by the caller keeps using them.  An entry is a few bytes per token."""
+    if stream is None:
+        stream = torch.cuda.current_stream().cuda_stream
+    key = (n_tokens, topk, dtype, device.type, device.index, int(stream))
     with _cache_lock:
         hit = _route_cache.get(key)
         if hit is None:
-            if len(_route_cache) > 64:
-                _route_cache.clear()
             hit = (torch.empty(n_tokens, topk, dtype=torch.int32, device=device),
                    torch.empty(n_tokens, topk, dtype=dtype, device=device))
             _route_cache[key] = hit

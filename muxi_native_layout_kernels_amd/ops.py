@@ -44,22 +44,54 @@ def _kind(t):
 
 
 # --------------------------------------------------------------- workspaces
-_ws_lock = threading.Lock()
-_ws = {}
+class WorkspacePool:
+    """Device scratch handed to the kernels as raw pointers (cross-workgroup K-split partials and their
+    arrival counters, the MoE alignment tables and intermediate).
+
+    * One buffer per (device, stream): two calls that run side by side on different streams never share
+      counters or partials.  Calls on one stream are ordered, so they can share.
+    * A buffer that has been handed out stays allocated for the life of the process.  A HIP graph captured
+      earlier replays with the pointer it was captured with; when a later call needs more room, a new, larger
+      buffer takes over for new calls and the old one is retired, not freed.
+    * `zero_prefix` bytes at the front are cleared when a buffer is created (the K-split kernels count
+      arrivals there and leave the counters at zero).
+    """
+
+    def __init__(self, min_bytes, zero_prefix=False):
+        self.min_bytes = int(min_bytes)
+        self.zero_prefix = zero_prefix
+        self._lock = threading.Lock()
+        self._live = {}
+        self._retired = []
+
+    def get(self, device, stream, nbytes, prefix_bytes=0):
+        key = (device.type, device.index, int(stream))
+        with self._lock:
+            buf = self._live.get(key)
+            if buf is None or buf.numel() < nbytes:
+                if buf is not None:
+                    self._retired.append(buf)
+                grown = 0 if buf is None else buf.numel() + buf.numel() // 2      # few retirements on a growing series
+                size = max(int(nbytes), self.min_bytes, grown)
+                buf = torch.empty(size, dtype=torch.uint8, device=device)
+                if self.zero_prefix and prefix_bytes:
+                    buf[:prefix_bytes].zero_()
+                self._live[key] = buf
+            return buf
+
+    def owned(self):
+        """Every buffer ever handed out (live and retired)."""
+        with self._lock:
+            return list(self._live.values()) + list(self._retired)
 
 
-def _workspace(device, nbytes, counter_bytes):
-    """Per-device scratch for cross-workgroup K splits.  The counter region at the
-    front is zeroed once at creation; the kernels leave it zero."""
-    key = (device.type, device.index)
-    with _ws_lock:
-        buf = _ws.get(key)
-        if buf is None or buf.numel() < nbytes:
-            size = max(int(nbytes), 1 << 22)
-            buf = torch.empty(size, dtype=torch.uint8, device=device)
-            buf[:counter_bytes].zero_()
-            _ws[key] = buf
-        return buf
+_gemm_pool = WorkspacePool(1 << 22, zero_prefix=True)
+_moe_pool = WorkspacePool(1 << 20)
+
+
+def _workspace(device, nbytes, counter_bytes, stream=None):
+    """Scratch for cross-workgroup K splits on `stream` (default: torch's current stream)."""
+    return _gemm_pool.get(device, _stream() if stream is None else stream, nbytes, counter_bytes)
 
 
 # ------------------------------------------------------------------ relayout
@@ -412,17 +444,8 @@ def batched_routed_activation_indexed_to_expert_block_indexed(batchSize, expertC
     return None
 
 
-_moe_ws = {}
-
-
-def _moe_workspace(device, nbytes):
-    key = (device.type, device.index)
-    with _ws_lock:
-        buf = _moe_ws.get(key)
-        if buf is None or buf.numel() < nbytes:
-            buf = torch.empty(max(int(nbytes), 1 << 20), dtype=torch.uint8, device=device)
-            _moe_ws[key] = buf
-        return buf
+def _moe_workspace(device, nbytes, stream=None):
+    return _moe_pool.get(device, _stream() if stream is None else stream, nbytes)
 
 
 def fused_experts_compute(experts_weights_matrix1, experts_weights_matrix2, activations, batch_size, expert_count,

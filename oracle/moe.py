@@ -102,7 +102,8 @@ def moe_expected(hidden, w1, w2, ids, wts, round_h_to=None, expert_map=None):
             a1, a2 = cache[e]
             proj = a1 @ x[t]
             g, u = proj[:inter], proj[inter:]
-            h = g / (1.0 + np.exp(-g)) * u
+            with np.errstate(over="ignore"):          # exp(-g) = inf for very negative g gives the right limit, -0
+                h = g / (1.0 + np.exp(-g)) * u
             if round_h_to is not None:
                 h = torch.from_numpy(h).to(torch.float32).to(round_h_to).to(torch.float64).numpy()
             y[t] += w_np[t, k] * (a2 @ h)

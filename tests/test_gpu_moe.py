@@ -132,24 +132,39 @@ def _pack_experts(w):
     return torch.stack([pack_a(w[e]) for e in range(w.shape[0])]).reshape(w.shape)
 
 
+def _rel_l2(got, want64):
+    g = got.detach().cpu().to(torch.float64).numpy()
+    return float(np.linalg.norm(g - want64) / max(np.linalg.norm(want64), 1e-30))
+
+
+def _outside(got, want64, rtol=RTOL, atol=ATOL):
+    """Fraction of elements the element-wise check would reject."""
+    g = got.detach().cpu().to(torch.float64).numpy()
+    return float((np.abs(g - want64) > atol + rtol * np.abs(want64)).mean())
+
+
 def _moe_case(mlk, T, E, K, H, I, dtype, seed, score="softmax", fp8=False, groups=None, bias=None, emap=None):
+    """One fused_moe call against the float64 statement.  Weights are drawn so that the outputs are of order
+    one (gate/up rows ~ N(0, 1/H), down rows ~ N(0, 4/I)): the tolerances then see every routed pair.  The
+    same check is run against the expected value with the last pick of every token removed and must reject it."""
     from muxi_native_layout_kernels_amd.moe_planC import fused_moe
     x = randn((T, H), dtype, 1.0, seed)
     logits = randn((T, E), dtype, 1.0, seed + 1)
+    std1, std2 = 1.0 / np.sqrt(H), 2.0 / np.sqrt(I)
     kw = {}
     if fp8:
         c1 = fp8_codes((E, 2 * I, H), seed + 2, std=1.0)
         c2 = fp8_codes((E, H, I), seed + 3, std=1.0)
         g = torch.Generator().manual_seed(seed + 4)
-        s1 = (torch.rand((E, 2 * I // 128, H // 128), generator=g) * 0.03 + 0.005).float()
-        s2 = (torch.rand((E, H // 128, I // 128), generator=g) * 0.03 + 0.005).float()
+        s1 = ((torch.rand((E, 2 * I // 128, H // 128), generator=g) + 0.5) * std1).float()
+        s2 = ((torch.rand((E, H // 128, I // 128), generator=g) + 0.5) * std2).float()
         w1u = omoe.dequant_experts(c1.numpy(), s1.numpy())
         w2u = omoe.dequant_experts(c2.numpy(), s2.numpy())
         w1p, w2p = _pack_experts(c1), _pack_experts(c2)
         kw = dict(w1_scale=s1.cuda(), w2_scale=s2.cuda(), block_shape=[128, 128], soft_fp8=True)
     else:
-        w1u = randn((E, 2 * I, H), dtype, 0.02, seed + 2)
-        w2u = randn((E, H, I), dtype, 0.02, seed + 3)
+        w1u = randn((E, 2 * I, H), dtype, std1, seed + 2)
+        w2u = randn((E, H, I), dtype, std2, seed + 3)
         w1p, w2p = _pack_experts(w1u), _pack_experts(w2u)
     n_groups, tk_groups = groups if groups else (1, 1)
     y = fused_moe(x.cuda(), w1p.cuda(), w2p.cuda(), logits.cuda(), K, True, use_grouped_topk=groups is not None,
@@ -160,6 +175,12 @@ def _moe_case(mlk, T, E, K, H, I, dtype, seed, score="softmax", fp8=False, group
     wts = orouter.renormalize(wts)
     want = omoe.moe_expected(x, w1u, w2u, ids, wts, round_h_to=dtype, expert_map=emap)
     assert_close(y, want, RTOL, ATOL, "fused_moe T=%d" % T)
+    assert _rel_l2(y, want) <= 1e-2
+    assert np.abs(want).mean() > 0.05, "the expected output carries no signal"
+    if K > 1 and emap is None:
+        # negative control: without the last pick of every token the same check must fail
+        fewer = omoe.moe_expected(x, w1u, w2u, ids[:, :K - 1], wts[:, :K - 1], round_h_to=dtype)
+        assert _outside(y, fewer) > 0.2 and _rel_l2(y, fewer) > 1e-2, "the check cannot see a dropped pick"
     return y
 
 
@@ -194,13 +215,17 @@ def test_fused_moe_expert_map(mlk):
     dtype = torch.bfloat16
     x = randn((T, H), dtype, 1.0, 1)
     logits = randn((T, E), dtype, 1.0, 2)
-    w1 = randn((4, 2 * I, H), dtype, 0.02, 3)
-    w2 = randn((4, H, I), dtype, 0.02, 4)
+    w1 = randn((4, 2 * I, H), dtype, 1.0 / np.sqrt(H), 3)
+    w2 = randn((4, H, I), dtype, 2.0 / np.sqrt(I), 4)
     y = fused_moe(x.cuda(), _pack_experts(w1).cuda(), _pack_experts(w2).cuda(), logits.cuda(), K, True,
                   experts_map=torch.as_tensor(emap).cuda())
     ids, wts = orouter.route(logits, 0, 1, 1, K)
     want = omoe.moe_expected(x, w1, w2, ids, orouter.renormalize(wts), round_h_to=dtype, expert_map=emap)
     assert_close(y, want, RTOL, ATOL, "expert map")
+    # negative control: treating the absent experts as present (weights of local expert e // 2) must fail the check
+    wrong = omoe.moe_expected(x, w1, w2, ids, orouter.renormalize(wts), round_h_to=dtype,
+                              expert_map=np.arange(8) // 2)
+    assert _outside(y, wrong) > 0.2
 
 
 @pytest.mark.parametrize("dtype,fp8,E,K,H,I", [
@@ -269,8 +294,8 @@ def test_fused_moe_single_token_expert_map(mlk):
     E, K, H, I = 8, 4, 256, 256
     dtype = torch.bfloat16
     emap = np.array([0, -1, 1, -1, 2, -1, 3, -1], dtype=np.int32)
-    w1 = randn((4, 2 * I, H), dtype, 0.02, 3)
-    w2 = randn((4, H, I), dtype, 0.02, 4)
+    w1 = randn((4, 2 * I, H), dtype, 1.0 / np.sqrt(H), 3)
+    w2 = randn((4, H, I), dtype, 2.0 / np.sqrt(I), 4)
     w1p, w2p = _pack_experts(w1).cuda(), _pack_experts(w2).cuda()
     for seed in range(4):
         x = randn((1, H), dtype, 1.0, 10 + seed)
@@ -304,8 +329,8 @@ def test_low_level_fused_experts_compute_signature(mlk):
     dtype = torch.float16
     x = randn((T, H), dtype, 1.0, 1).cuda()
     logits = randn((T, E), dtype, 1.0, 2).cuda()
-    w1u = randn((E, 2 * I, H), dtype, 0.02, 3)
-    w2u = randn((E, H, I), dtype, 0.02, 4)
+    w1u = randn((E, 2 * I, H), dtype, 1.0 / np.sqrt(H), 3)
+    w2u = randn((E, H, I), dtype, 2.0 / np.sqrt(I), 4)
     w1, w2 = _pack_experts(w1u).cuda(), _pack_experts(w2u).cuda()
     ids = torch.empty(T, K, dtype=torch.int32, device="cuda")
     wts = torch.empty(T, K, dtype=dtype, device="cuda")
@@ -325,9 +350,27 @@ def test_low_level_fused_experts_compute_signature(mlk):
     assert int(pn.item()) == oalign.align_tokens(ids.cpu().numpy(), E)["padded_num_blocks"]
 
 
-@pytest.mark.parametrize("T", [1, 16])
+class _Lazy:
+    """Per-expert weights fetched on demand (only the experts the sampled tokens use reach the host)."""
+
+    def __init__(self, fetch, shape):
+        self.fetch, self.shape, self.cache = fetch, shape, {}
+
+    def __getitem__(self, e):
+        if e not in self.cache:
+            self.cache[e] = self.fetch(e)
+        return self.cache[e]
+
+
+def _sample_tokens(T):
+    return list(range(T)) if T <= 4 else sorted({0, T // 2 + 1, T - 1})
+
+
+@pytest.mark.parametrize("T", [1, 16, 64, 256])
 def test_fused_moe_mixtral_shape(mlk, T):
-    """E=8, top-2, H=4096, I=14336 at full size; the oracle only evaluates the selected experts."""
+    """E=8, top-2, H=4096, I=14336, bf16 weights ~ N(0, 0.02) at full size; the oracle evaluates sampled tokens
+    (from different token blocks) on the experts they select.  64 and 256 tokens run the row-shared kernels
+    and the combine kernel."""
     from muxi_native_layout_kernels_amd.moe_planC import fused_moe
     E, K, H, I = 8, 2, 4096, 14336
     dtype = torch.bfloat16
@@ -339,17 +382,143 @@ def test_fused_moe_mixtral_shape(mlk, T):
     w1p = mlk.pack_layout_a(w1u).view(E, 2 * I, H)
     w2p = mlk.pack_layout_a(w2u).view(E, H, I)
     y = fused_moe(x.cuda(), w1p, w2p, logits.cuda(), K, True)
+    y2 = fused_moe(x.cuda(), w1p, w2p, logits.cuda(), K, True)
+    assert torch.equal(y, y2)
     ids, wts = orouter.route(logits, 0, 1, 1, K)
     wts = orouter.renormalize(wts)
-    tok = list(range(T)) if T <= 4 else [0, T // 2, T - 1]    # bound the float64 work on the host
-    w1c, w2c = {}, {}
-    for t in tok:
-        for e in ids[t].tolist():
-            if e not in w1c:
-                w1c[e], w2c[e] = w1u[e].cpu(), w2u[e].cpu()
-    class Lazy:
-        def __init__(self, d, shape): self.d, self.shape = d, shape
-        def __getitem__(self, e): return self.d[e]
-    want = omoe.moe_expected(x[tok], Lazy(w1c, (E, 2 * I, H)), Lazy(w2c, (E, H, I)), ids[tok], wts[tok],
-                             round_h_to=dtype)
+    tok = _sample_tokens(T)
+    want = omoe.moe_expected(x[tok], _Lazy(lambda e: w1u[e].cpu(), (E, 2 * I, H)), _Lazy(lambda e: w2u[e].cpu(), (E, H, I)),
+                             ids[tok], wts[tok], round_h_to=dtype)
     assert_close(y[tok], want, RTOL, ATOL, "mixtral T=%d" % T)
+    assert _rel_l2(y[tok], want) <= 1e-2 and np.abs(want).mean() > 0.3
+    fewer = omoe.moe_expected(x[tok], _Lazy(lambda e: w1u[e].cpu(), (E, 2 * I, H)),
+                              _Lazy(lambda e: w2u[e].cpu(), (E, H, I)), ids[tok][:, :1], wts[tok][:, :1], round_h_to=dtype)
+    assert _outside(y[tok], fewer) > 0.2
+    # every token is finite and of the expected size (the sampled ones are checked exactly)
+    yn = y.float()
+    assert torch.isfinite(yn).all() and 0.2 < float(yn.abs().mean()) < 20.0
+
+
+@pytest.mark.parametrize("T,unit_scales", [(1, False), (16, True), (16, False), (64, False), (256, False)])
+def test_fused_moe_mixtral_shape_soft_fp8(mlk, T, unit_scales):
+    """The soft-FP8 variant of the same layer: e4m3 bytes from N(0, 1) * 16 clipped to +-448, one fp32 scale per
+    128 x 128 block (all ones as the benchmark runs it, or random factors around 1e-3)."""
+    from muxi_native_layout_kernels_amd.moe_planC import fused_moe
+    from oracle import softfp8
+    E, K, H, I = 8, 2, 4096, 14336
+    dtype = torch.bfloat16
+    x = randn((T, H), dtype, 1.0, 3025)
+    logits = randn((T, E), dtype, 1.0, 3026)
+    g = torch.Generator(device="cuda").manual_seed(3027)
+    c1 = (torch.randn((E, 2 * I, H), generator=g, device="cuda") * 16).clamp_(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+    c2 = (torch.randn((E, H, I), generator=g, device="cuda") * 16).clamp_(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+    if unit_scales:
+        s1 = torch.ones((E, 2 * I // 128, H // 128), dtype=torch.float32, device="cuda")
+        s2 = torch.ones((E, H // 128, I // 128), dtype=torch.float32, device="cuda")
+    else:
+        s1 = (torch.rand((E, 2 * I // 128, H // 128), generator=g, device="cuda") + 0.5) * 1.0e-3
+        s2 = (torch.rand((E, H // 128, I // 128), generator=g, device="cuda") + 0.5) * 1.3e-3
+    w1p = mlk.pack_layout_a(c1).view(E, 2 * I, H)
+    w2p = mlk.pack_layout_a(c2).view(E, H, I)
+    y = fused_moe(x.cuda(), w1p, w2p, logits.cuda(), K, True, w1_scale=s1, w2_scale=s2, block_shape=[128, 128],
+                  soft_fp8=True)
+    y2 = fused_moe(x.cuda(), w1p, w2p, logits.cuda(), K, True, w1_scale=s1, w2_scale=s2, block_shape=[128, 128],
+                   soft_fp8=True)
+    assert torch.equal(y, y2)
+    ids, wts = orouter.route(logits, 0, 1, 1, K)
+    wts = orouter.renormalize(wts)
+    tok = _sample_tokens(T)
+    w1l = _Lazy(lambda e: softfp8.dequant_weight_f32(c1[e].cpu().numpy(), s1[e].cpu().numpy()), (E, 2 * I, H))
+    w2l = _Lazy(lambda e: softfp8.dequant_weight_f32(c2[e].cpu().numpy(), s2[e].cpu().numpy()), (E, H, I))
+    want = omoe.moe_expected(x[tok], w1l, w2l, ids[tok], wts[tok], round_h_to=dtype)
+    # outputs are huge with unit scales (weights ~ N(0, 16)): the check is relative, the absolute term is scaled up
+    scale = max(1.0, float(np.abs(want).mean()))
+    assert_close(y[tok], want, RTOL, ATOL * scale, "mixtral soft-FP8 T=%d" % T)
+    assert _rel_l2(y[tok], want) <= 1e-2
+    fewer = omoe.moe_expected(x[tok], w1l, w2l, ids[tok][:, :1], wts[tok][:, :1], round_h_to=dtype)
+    assert _outside(y[tok], fewer, RTOL, ATOL * scale) > 0.2
+    assert torch.isfinite(y.float()).all()
+
+
+# -------------------------------------------------------------- the reference's own test grid
+def _pack_view_permute(w):
+    """The packing loop of the reference's tests (test_muxi_moe.py:73-81) for all experts at once."""
+    e, n, k = w.shape
+    return w.view(e, n // 16, 16, k // 8, 8).permute(0, 1, 3, 2, 4).contiguous().view(e, n, k)
+
+
+@pytest.mark.parametrize("m", [8, 16, 64, 256, 2048])
+@pytest.mark.parametrize("n,k,e", [(256, 7168, 256), (768, 2048, 128)])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_reference_grid(mlk, m, n, k, e, dtype):
+    """benchmark_and_test/test_muxi_moe.py:14-111 at its own shapes and with its own recipe: top-8, sigmoid, 8 groups
+    of which 4 are kept, renormalised, `rand / 100` activations, `rand / 10` weights, `rand` logits, compared with
+    the pure-torch MoE run on the GPU in the same dtype to atol 0.1 / rtol 0.05.  On top of that, sampled tokens
+    are checked against the float64 statement with the router's own tie rule to rtol = atol = 1e-2."""
+    from muxi_native_layout_kernels_amd.moe_planC import fused_moe
+    from muxi_native_layout_kernels_amd import utils
+    topk = 8
+    torch.manual_seed(2025)
+    a = torch.rand((m, k), device="cuda", dtype=dtype) / 100
+    w1 = torch.rand((e, 2 * n, k), device="cuda", dtype=dtype) / 10
+    w2 = torch.rand((e, k, n), device="cuda", dtype=dtype) / 10
+    score = torch.rand((m, e), device="cuda", dtype=dtype)
+    out = fused_moe(a, _pack_view_permute(w1), _pack_view_permute(w2), score, topk, renormalize=True,
+                    use_grouped_topk=True, num_expert_group=8, topk_group=4, gating_bias=None, score_func="sigmoid")
+    ref = utils.fused_moe(a.clone(), w1, w2, score, topk, 8, 4, global_num_experts=e, renormalize=True,
+                          e_score_correction_bias=None, score_func="sigmoid")
+    torch.testing.assert_close(out, ref, atol=0.1, rtol=0.05)
+    assert float(ref.float().abs().mean()) > 1.0            # the recipe gives outputs far above the tolerance
+    # float64 statement on sampled tokens
+    tok = sorted({0, m // 2, m - 1})
+    ids, wts = orouter.route(score[tok].cpu(), 1, 8, 4, topk)      # rows are routed independently
+    wts = orouter.renormalize(wts)
+    w1l = _Lazy(lambda i: w1[i].cpu(), (e, 2 * n, k))
+    w2l = _Lazy(lambda i: w2[i].cpu(), (e, k, n))
+    want = omoe.moe_expected(a[tok].cpu(), w1l, w2l, ids, wts, round_h_to=dtype)
+    assert_close(out[tok], want, RTOL, ATOL, "reference grid m=%d" % m)
+    fewer = omoe.moe_expected(a[tok].cpu(), w1l, w2l, ids[:, :topk - 1], wts[:, :topk - 1], round_h_to=dtype)
+    assert _outside(out[tok], fewer) > 0.5
+
+
+@pytest.mark.parametrize("m", [8, 64, 244, 256, 2048])
+@pytest.mark.parametrize("n,k,e", [(256, 7168, 256), (768, 2048, 128)])
+def test_reference_grid_soft_fp8(mlk, m, n, k, e):
+    """benchmark_and_test/test_muxi_moe_softfp8.py:57-129: the same grid with float8_e4m3fn weights and
+    `rand * 2` block scales, expected value from `scale_whole_tensor` + the pure-torch MoE in bf16."""
+    from muxi_native_layout_kernels_amd.moe_planC import fused_moe
+    from muxi_native_layout_kernels_amd import utils
+    from oracle import softfp8
+    topk, dtype = 8, torch.bfloat16
+    torch.manual_seed(2025)
+    a = torch.rand((m, k), device="cuda", dtype=dtype) / 100
+    w1 = (torch.rand((e, 2 * n, k), device="cuda", dtype=dtype) / 10).to(torch.float8_e4m3fn)
+    w2 = (torch.rand((e, k, n), device="cuda", dtype=dtype) / 10).to(torch.float8_e4m3fn)
+    w1_scale = torch.rand((e, 2 * n // 128, k // 128), device="cuda", dtype=torch.float32) * 2
+    w2_scale = torch.rand((e, k // 128, n // 128), device="cuda", dtype=torch.float32) * 2
+    score = torch.rand((m, e), device="cuda", dtype=dtype)
+    out = fused_moe(a, _pack_view_permute(w1.view(torch.uint8)), _pack_view_permute(w2.view(torch.uint8)), score, topk,
+                    renormalize=True, use_grouped_topk=True, num_expert_group=8, topk_group=4, gating_bias=None,
+                    score_func="sigmoid", w1_scale=w1_scale, w2_scale=w2_scale, block_shape=[128, 128], soft_fp8=True)
+    ref = utils.fused_moe(a.clone(), utils.scale_whole_tensor(w1, w1_scale), utils.scale_whole_tensor(w2, w2_scale),
+                          score, topk, 8, 4, global_num_experts=e, renormalize=True, e_score_correction_bias=None,
+                          score_func="sigmoid")
+    torch.testing.assert_close(out, ref, atol=0.1, rtol=0.05)
+    assert float(ref.float().abs().mean()) > 1.0
+    tok = sorted({0, m // 2, m - 1})
+    ids, wts = orouter.route(score[tok].cpu(), 1, 8, 4, topk)
+    wts = orouter.renormalize(wts)
+    c1, c2 = w1.view(torch.uint8), w2.view(torch.uint8)
+    w1l = _Lazy(lambda i: softfp8.dequant_weight_f32(c1[i].cpu().numpy(), w1_scale[i].cpu().numpy()), (e, 2 * n, k))
+    w2l = _Lazy(lambda i: softfp8.dequant_weight_f32(c2[i].cpu().numpy(), w2_scale[i].cpu().numpy()), (e, k, n))
+    want = omoe.moe_expected(a[tok].cpu(), w1l, w2l, ids, wts, round_h_to=dtype)
+    assert_close(out[tok], want, RTOL, ATOL, "reference grid soft-FP8 m=%d" % m)
+
+
+@pytest.mark.parametrize("T", [171, 172, 244, 256, 500])
+def test_fused_moe_soft_fp8_many_experts_near_a_full_pass(mlk, T):
+    """256 experts, top-8, soft-FP8 with 170 to 256 tokens in a pass: one token block per task, so the decode down
+    kernel runs with an output tile of up to 256 tokens; the rows per wave are chosen so that it fits the LDS."""
+    E = 256
+    bias = randn((E,), torch.bfloat16, 0.05, 78).abs()
+    _moe_case(mlk, T, E, 8, 512, 256, torch.bfloat16, 1500 + T, score="sigmoid", groups=(8, 4), bias=bias, fp8=True)

@@ -89,3 +89,87 @@ def test_panel_kernel_default_shape():
     assert sel._gemm_default_rowmajor(11008, 64, 4096)[0] == 1      # the narrow kernels up to 64 tokens
     assert sel._gemm_default_rowmajor(11008, 512, 4096 + 64)[0] == 2  # K is no multiple of 128
     assert sel._gemm_default(11008, 512, 4096)[0] == 2              # native operands never get the panel kernel
+
+
+def test_workspace_pool_never_frees_what_it_handed_out():
+    """A larger request gets a new buffer; the earlier one stays owned (a captured graph may still use its
+    address).  Streams do not share buffers, repeated requests on one stream do."""
+    pool = ops.WorkspacePool(1024, zero_prefix=True)
+    cpu = torch.device("cpu")
+    a = pool.get(cpu, 0, 1000, 64)
+    ptr_a = a.data_ptr()
+    assert a.numel() >= 1024 and not a[:64].any()
+    assert pool.get(cpu, 0, 512, 64) is a                     # fits: same buffer
+    b = pool.get(cpu, 0, 1 << 16, 64)
+    assert b is not a and b.numel() >= 1 << 16 and not b[:64].any()
+    assert pool.get(cpu, 0, 1000, 64) is b                    # new calls use the larger one
+    c = pool.get(cpu, 7, 1000, 64)                            # another stream: its own buffer
+    assert c is not a and c is not b
+    owned = {t.data_ptr() for t in pool.owned()}
+    assert {ptr_a, b.data_ptr(), c.data_ptr()} <= owned
+    a.fill_(3)                                                # still valid memory of ours
+    assert int(a[5]) == 3
+    # growth is geometric, so a slowly growing series of shapes retires few buffers
+    for n in range(1 << 16, 1 << 18, 4096):
+        pool.get(cpu, 0, n, 64)
+    assert len(pool.owned()) <= 8
+
+
+def test_routing_buffers_are_kept_for_every_shape_and_stream():
+    from muxi_native_layout_kernels_amd import moe_planC
+    cpu = torch.device("cpu")
+    first = moe_planC._routing_buffers(3, 2, torch.bfloat16, cpu, stream=0)
+    ptr = first[0].data_ptr()
+    for t in range(4, 140):                                   # many other shapes must not evict it
+        moe_planC._routing_buffers(t, 2, torch.bfloat16, cpu, stream=0)
+    again = moe_planC._routing_buffers(3, 2, torch.bfloat16, cpu, stream=0)
+    assert again[0].data_ptr() == ptr and again[1] is first[1]
+    other = moe_planC._routing_buffers(3, 2, torch.bfloat16, cpu, stream=5)
+    assert other[0].data_ptr() != ptr
+
+
+def _plan(T, E, K, H, I, kind):
+    import ctypes
+    out = (ctypes.c_int32 * 8)()
+    rc = _lib.load().mlk_moe_plan(T, E, K, H, I, kind, ctypes.addressof(out))
+    assert rc == 0
+    return dict(path=out[0], cb=out[1], max_tasks=out[2], down_r=out[3], down_slices=out[4], down_wk=out[5],
+                down_lds=out[6], static_lds=out[7])
+
+
+@pytest.mark.parametrize("kind", [1, 2])
+@pytest.mark.parametrize("E,K,H,I", [(256, 8, 7168, 256), (256, 8, 256, 128), (128, 8, 2048, 768), (8, 2, 4096, 14336),
+                                     (64, 6, 1024, 512)])
+def test_moe_plan_fits_the_workgroup_lds_for_every_token_count(E, K, H, I, kind):
+    """Every pass of 1..256 tokens (also the remainder passes of longer inputs) must get a down-projection
+    shape whose LDS fits the 64 KiB a workgroup gets by default, with at least four waves whenever more
+    than one row group per wave was chosen."""
+    for T in range(1, 257):
+        p = _plan(T, E, K, H, I, kind)
+        assert p["path"] in (0, 1, 2, 3) and p["cb"] in (1, 2, 3, 4, 6, 8)
+        if p["path"] in (1, 2):
+            assert p["down_lds"] + p["static_lds"] <= 64 * 1024, (T, p)
+            assert p["down_wk"] >= 1 and p["down_lds"] == p["down_wk"] * p["down_r"] * p["cb"] * 1024 + T * 16 * p["down_r"] * 4
+            if p["down_r"] > 1:
+                assert p["down_wk"] >= 4 and p["cb"] == 1 and p["down_slices"] == p["down_r"], (T, p)
+                assert (H // 16) % p["down_r"] == 0 and (I // 32) % p["down_r"] == 0
+        if p["path"] == 3:
+            assert p["cb"] >= 2 and (I // 32) % (p["down_slices"] * (2 if p["cb"] > 4 else 4)) == 0
+        assert p["path"] != 0 or T == 1
+
+
+def test_moe_plan_known_cases():
+    # soft-FP8, 256 experts, top-8 (the DeepSeek configuration): 4 row groups per wave while the output tile
+    # fits, 2 from 172 tokens up (the tile of 4 row groups would leave fewer than four waves)
+    assert _plan(16, 256, 8, 7168, 256, 2)["down_r"] == 4
+    assert _plan(171, 256, 8, 7168, 256, 2)["down_r"] == 4
+    assert _plan(172, 256, 8, 7168, 256, 2)["down_r"] == 2
+    assert _plan(244, 256, 8, 7168, 256, 2)["down_r"] == 2
+    assert _plan(244, 256, 8, 7168, 256, 2)["path"] == 2
+    # Mixtral shape: one token -> GeMV kernels; 16 tokens -> in-kernel alignment; 64 and 256 -> row-shared kernels
+    assert _plan(1, 8, 2, 4096, 14336, 1)["path"] == 0
+    assert _plan(16, 8, 2, 4096, 14336, 1)["path"] == 1
+    assert _plan(64, 8, 2, 4096, 14336, 1)["path"] == 3
+    assert _plan(256, 8, 2, 4096, 14336, 1)["path"] == 3
+    # 500 tokens run as 256 + 244: the plan of the first pass is what the query reports
+    assert _plan(500, 256, 8, 7168, 256, 2) == _plan(256, 256, 8, 7168, 256, 2)
