@@ -176,6 +176,20 @@ int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, int n, int k
 size_t mlk_gemm_workspace_bytes(int m, int n, int p1, int p3);
 size_t mlk_gemm_counter_bytes(void);
 
+/* mlk_gemm_layout_a for callers that can neither allocate device memory nor bring a workspace (code under
+ * HIP graph capture, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference.  Same arguments, kernels and results as mlk_gemm_layout_a; the scratch of a K split across
+ * workgroups (p3 > 1) lives in a device array built into the library, mlk_gemm_noalloc_scratch_bytes() =
+ * 16 MiB per GPU, held until the process ends.  A call whose mlk_gemm_workspace_bytes(m, n, p1, p3) exceeds
+ * that returns MLK_ERR_WORKSPACE and launches nothing.  The call allocates and frees nothing.  All calls on
+ * one GPU share the array: calls that may overlap (different streams, or graphs replayed side by side) race;
+ * order them on one stream.  The first call on a GPU looks up the array's address and clears the counter
+ * region with a small kernel on `stream`. */
+int mlk_gemm_layout_a_noalloc(const void *a, const void *b, void *c, int m, int n, int k, int a_kind, int x_kind,
+                              int b_mode, int c_mode, float alpha, const void *bias, const float *scale,
+                              int kernel_id, int p1, int p2, int p3, void *stream);
+size_t mlk_gemm_noalloc_scratch_bytes(void);
+
 /* ----------------------------------------------------------------------- MoE */
 
 /* Router: scores (score_fun 0 = softmax, 1 = sigmoid), optional correction

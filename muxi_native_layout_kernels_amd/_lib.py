@@ -30,6 +30,9 @@ SIGNATURES = {
     "mlk_gemm_layout_a": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
                                   c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p, c_size_t,
                                   c_void_p]),
+    "mlk_gemm_layout_a_noalloc": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
+                                          c_int, c_float, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
+    "mlk_gemm_noalloc_scratch_bytes": (c_size_t, []),
     "mlk_gemm_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int]),
     "mlk_gemm_counter_bytes": (c_size_t, []),
     "mlk_fused_routing_gate": (c_int, [c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void_p, c_int,

@@ -1,10 +1,49 @@
 // Host entry points of the narrow GeMM (the kernels live in mlk_gemm_kernels.cuh and are
 // instantiated per operand type in mlk_gemm_f16.hip, mlk_gemm_bf16.hip and mlk_gemm_fp8.hip).
+#include <atomic>
+#include <mutex>
+
 #include "mlk_gemm_kernels.cuh"
 
 namespace mlk {
 
 constexpr size_t kCounterBytes = 64 * 1024;
+
+// Scratch of mlk_gemm_layout_a_noalloc(): arrival counters and fp32 partials of the cross-workgroup K splits,
+// for callers that can neither allocate nor pass a workspace.  One copy per GPU, held until the process ends.
+constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+static std::atomic<void *> g_scratch_ptr[64];     // per device: the array's address on that device
+static std::mutex g_scratch_mutex;
+
+__global__ void __launch_bounds__(256) zero_words_kernel(uint32_t *p, int n) {
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0u;
+}
+
+// Address of `scratch` on the current device.  On the first call on a device the address is looked up and
+// the counter region is cleared by a small kernel on `s` (ordered before the caller's launches on `s`).
+static int static_scratch(void **out, hipStream_t s) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));
+    if (dev < 0 || dev >= 64) return fail(MLK_ERR_INVALID, "gemm: device index above 63");
+    void *ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (ptr == nullptr) {
+        std::lock_guard<std::mutex> lock(g_scratch_mutex);
+        ptr = g_scratch_ptr[dev].load(std::memory_order_acquire);
+        if (ptr == nullptr) {
+            e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+            if (e != hipSuccess || ptr == nullptr)
+                return fail(MLK_ERR_LAUNCH, e != hipSuccess ? hipGetErrorString(e) : "gemm: no address for the static scratch");
+            zero_words_kernel<<<16, 256, 0, s>>>((uint32_t *)ptr, (int)(kCounterBytes / 4));
+            e = hipGetLastError();
+            if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));
+            g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+        }
+    }
+    *out = ptr;
+    return MLK_OK;
+}
 
 // Experiment switches (mlk_set_tunable): [0] rotate the k-tile order per row tile,
 // [1] stage row-major activations through LDS, [2]..[5] and [7] shape the fused MoE kernels
@@ -132,4 +171,23 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
         if (rc != MLK_OK) return rc;
     }
     return MLK_OK;
+}
+
+extern "C" size_t mlk_gemm_noalloc_scratch_bytes(void) { return kStaticScratchBytes; }
+
+extern "C" int mlk_gemm_layout_a_noalloc(const void *a, const void *b, void *c, int m, int n, int k, int a_kind,
+                                         int x_kind, int b_mode, int c_mode, float alpha, const void *bias,
+                                         const float *scale, int kernel_id, int p1, int p2, int p3, void *stream) {
+    void *ws = nullptr;
+    if (p3 > 1) {
+        MLK_REQUIRE(m >= 0 && n >= 0 && n % 16 == 0, "gemm: N % 16 must be 0");
+        if (mlk_gemm_workspace_bytes(m, n, p1, p3) > kStaticScratchBytes)
+            return fail(MLK_ERR_WORKSPACE,
+                        "gemm: this K split needs more than the 16 MiB of built-in scratch; use fewer splits (p3) "
+                        "or mlk_gemm_layout_a with a caller-owned workspace");
+        const int rc = static_scratch(&ws, (hipStream_t)stream);
+        if (rc != MLK_OK) return rc;
+    }
+    return mlk_gemm_layout_a(a, b, c, m, n, k, a_kind, x_kind, b_mode, c_mode, alpha, bias, scale, kernel_id, p1, p2,
+                             p3, ws, ws ? kStaticScratchBytes : 0, stream);
 }
