@@ -1,29 +1,36 @@
 #!/usr/bin/env python3
 """Benchmark of the native-layout hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--case TEXT] [--no-cpu]
 
 Prints ONE JSON line.  The headline workload is the fp16 narrow GeMM of the
 second benchmark configuration (`gemm_layoutA`, weights 11008 x 4096 in
 layout-A, 16 tokens); one step is one call.  Inputs are synthetic, seeded and
 resident in HBM before the timed region.  Every call of a timed region reads a
 different weight copy (enough copies to exceed the 256 MiB Infinity Cache), so
-the bandwidth is HBM bandwidth.  The K timed calls are replayed from one HIP
-graph, bracketed by HIP events on the stream that runs them.  Before the timed
-replay come the W warm-up calls and un-timed replays of the same graph for at
-least 20 ms: the graph capture leaves the GPU idle, and the first replays after
-an idle period run several percent below the steady state this measures.
+the bandwidth is HBM bandwidth.
 
-`per_config` in the same line holds the other configurations (bf16 / soft-FP8
-GeMV, the M sweep, the native-layout chain and the fused MoE layer) with
-microseconds per call, achieved GB/s of algorithmic bytes and the fraction of
-the 8 TB/s HBM peak.  `cpu_baseline` is the reference's CPU-runnable path (a
-library linear on the un-packed weights in the same dtype) timed on the host
-cores on a bounded sample.
+Timing protocol: the K calls are recorded into one HIP graph.  After the W
+warm-up calls and un-timed replays of the graph for at least 20 ms (the capture
+leaves the GPU idle and the first replays after an idle period run several
+percent below the steady state), the graph is replayed five times, each replay
+(exactly K calls) bracketed by HIP events on the stream that runs it.  The
+headline value comes from the first timed replay; the median and the minimum
+of the five are reported beside it, and for every other configuration.
+
+`per_config` holds the other configurations (bf16 / soft-FP8 GeMV, the M sweep,
+the native-layout chain, the relayout kernels and the fused MoE layer) with
+microseconds per call, achieved GB/s of algorithmic bytes, the fraction of the
+8 TB/s HBM peak, a pure-read launch of the same weight bytes as a yardstick
+where the weights are small, HBM traffic from hardware counters where a
+profile under profiles/ holds it, and the CPU baseline of that configuration:
+the reference's CPU-runnable torch path (a library linear on the un-packed
+weights, or its dense MoE loop) timed on the host cores on a bounded sample.
 """
 import argparse
 import json
 import os
+import statistics
 import sys
 import time
 
@@ -34,6 +41,7 @@ if ROOT not in sys.path:
 HBM_PEAK_GBPS = 8000.0
 MFMA_PEAK_TFLOPS = 2500.0      # dense fp16 / bf16 (soft-FP8 weights are widened to bf16 before the product)
 MALL_BYTES = 256 << 20
+TIMED_REPLAYS = 5
 
 
 def main():
@@ -42,10 +50,10 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--quick", action="store_true", help="headline workload only")
-    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--case", default=None,
                     help="besides the headline, run only the per-configuration cases whose name contains this text "
-                         "(for profiling one kernel)")
+                         "(several texts separated by commas; for profiling single kernels)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain copy kernel of known size (256 MiB in, 256 MiB out) so that "
                          "hardware byte counters can be scaled against it")
@@ -64,6 +72,16 @@ def main():
     torch.cuda.set_device(dev)
     gen = torch.Generator(device=dev).manual_seed(2025)
     DT = {0: torch.float16, 1: torch.bfloat16}
+    cores = torch.get_num_threads()
+    host_cpus = os.cpu_count() or 0
+
+    traffic_table = {}
+    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
+    if os.path.exists(tpath):
+        try:
+            traffic_table = json.load(open(tpath))
+        except (OSError, ValueError):
+            traffic_table = {}
 
     def copies_for(nbytes):
         return int(max(2, min(24, (3 * MALL_BYTES + nbytes - 1) // nbytes)))
@@ -80,13 +98,16 @@ def main():
                 out.append((torch.randn((n // 16, k // 8, 16, 8), generator=gen, device=dev) * 0.02).to(DT[kind]))
         return out
 
+    bench_stream = torch.cuda.Stream()      # every timed region runs on this one stream
+
     def settle_replays(steps):
         return 1 + max(1, int(0.02 / (steps * 20e-6)))      # >= 20 ms at 20 us per call
 
-    def run_graph(calls, steps, warmup):
-        """Replay `steps` calls (cycling through `calls`) from one HIP graph; returns
-        (microseconds per call from HIP events on the launching stream, wall seconds of the timed region)."""
-        stream = torch.cuda.Stream()
+    def run_graph(calls, steps, warmup, reps=TIMED_REPLAYS):
+        """Replay `steps` calls (cycling through `calls`) from one HIP graph, `reps` times, each replay between
+        HIP events on the launching stream.  Returns microseconds per call of the first timed replay, the median
+        and the minimum over the replays, and the wall seconds of the first timed replay."""
+        stream = bench_stream
         with torch.cuda.stream(stream):
             for i in range(max(warmup, 3)):
                 calls[i % len(calls)]()
@@ -95,24 +116,120 @@ def main():
             with torch.cuda.graph(graph, stream=stream):
                 for i in range(steps):
                     calls[i % len(calls)]()
-            # un-timed replays until the clocks have settled: right after the (CPU-bound, GPU-idle) graph
-            # capture the first replays run several percent slower than the steady state
             for _ in range(settle_replays(steps)):
                 graph.replay()
             torch.cuda.synchronize()
-            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            t0 = time.perf_counter()
-            e0.record()
-            graph.replay()
-            e1.record()
-            torch.cuda.synchronize()
-            wall = time.perf_counter() - t0
-            us = e0.elapsed_time(e1) * 1e3 / steps
-        return us, wall
+            us, wall = [], None
+            for _ in range(reps):
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                t0 = time.perf_counter()
+                e0.record()
+                graph.replay()
+                e1.record()
+                torch.cuda.synchronize()
+                if wall is None:
+                    wall = time.perf_counter() - t0
+                us.append(e0.elapsed_time(e1) * 1e3 / steps)
+        return dict(us=us[0], us_median=statistics.median(us), us_min=min(us), wall=wall)
 
-    def gemv_case(name, n, k, kind, steps, warmup):
+    def finish(name, t, algo, **extra):
+        row = dict(name=name, us=t["us"], us_median=t["us_median"], us_min=t["us_min"], bytes=algo,
+                   gbps=algo / t["us"] / 1e3, frac=algo / t["us"] / 1e3 / HBM_PEAK_GBPS, wall=t["wall"])
+        row.update(extra)
+        if name in traffic_table:
+            row["traffic"] = traffic_table[name]
+            row["traffic_over_algorithmic"] = traffic_table[name] / algo
+        return row
+
+    def read_only_us(nbytes, steps, shapes=((512, 1024), (1024, 512), (256, 2048), (512, 512), (1024, 256))):
+        """One launch that only reads `nbytes` (rotating copies, GeMV access pattern): best us per launch."""
+        nbytes -= nbytes % 4096
+        bufs = [torch.randint(0, 255, (nbytes,), dtype=torch.uint8, device=dev) for _ in range(copies_for(nbytes))]
+        best = None
+        for block, wgs in shapes:
+            if (nbytes // 1024) % wgs:
+                continue
+
+            def mk(b):
+                def call():
+                    _lib.check(lib.mlk_stream_read(b.data_ptr(), nbytes, block, wgs, 0,
+                                                   torch.cuda.current_stream().cuda_stream), "stream_read")
+                return call
+            t = run_graph([mk(b) for b in bufs], steps, 5, reps=3)
+            best = t["us_median"] if best is None else min(best, t["us_median"])
+        return best
+
+    # ------------------------------------------------------------------ CPU baselines
+    def cpu_time(fn, budget_s=0.8, min_reps=3, max_reps=50):
+        for _ in range(2):
+            fn()
+        reps, t0 = 0, time.perf_counter()
+        while reps < min_reps or (time.perf_counter() - t0 < budget_s and reps < max_reps):
+            fn()
+            reps += 1
+        return (time.perf_counter() - t0) / reps, reps
+
+    def cpu_linear(n, k, m, kind, rows, native=False):
+        """The reference's CPU-runnable path for one GeMV / GeMM configuration on the first `rows` weight rows:
+        a library linear on the un-packed weights in the configuration's dtype; soft-FP8 weights are first
+        widened and scaled per block in bf16 (done once, outside the timing, as the reference's scripts do);
+        the native chain adds the view/permute pack and un-pack of the output."""
+        if args.no_cpu:
+            return None
+        from oracle import gemm as ogemm
+        rows = min(rows, n)
+        g = torch.Generator().manual_seed(2025)
+        dt = torch.bfloat16 if kind == 2 else DT[kind]
+        if kind == 2:
+            codes = (torch.randn((rows, k), generator=g) * 16).clamp_(-448, 448).to(torch.float8_e4m3fn).view(torch.uint8)
+            w = ogemm.torch_path_softfp8_weight(codes, torch.ones(((rows + 127) // 128, (k + 127) // 128)))
+        else:
+            w = (torch.randn((rows, k), generator=g) * 0.02).to(dt)
+        b = torch.randn((m, k), generator=g).to(dt)
+
+        def fn():
+            c = ogemm.torch_path_linear(w, b)
+            if native:
+                c_nat = ogemm.layout_c_of(c)
+                c = c_nat.view(rows // 32, m // 16, 4, 16, 8).permute(1, 3, 0, 2, 4).contiguous().view(m, rows)
+            return c
+        dt_s, reps = cpu_time(fn)
+        sample_bytes = rows * k * (1 if kind == 2 else 2) + m * k * 2 + m * rows * 2
+        return dict(value=round(sample_bytes / dt_s / 1e9, 3), unit="GB/s", us_scaled_to_full=round(dt_s * 1e6 * n / rows, 1),
+                    cores=cores, kind="port",
+                    sample="torch linear in %s on the first %d of %d un-packed weight rows, M=%d, %d reps, %.3f ms each; "
+                           "host has %d logical CPUs" % (str(dt).replace("torch.", ""), rows, n, m, reps, dt_s * 1e3,
+                                                          host_cpus))
+
+    cpu_moe_w = {}
+
+    def cpu_moe(T, slab=8):
+        """The reference's dense torch MoE (all 8 experts on every token) on 1/slab of the intermediate size."""
+        if args.no_cpu:
+            return None
+        from oracle import moe as omoe
+        E, K, H, I = 8, 2, 4096, 14336 // slab
+        g = torch.Generator().manual_seed(2025)
+        if "w" not in cpu_moe_w:
+            cpu_moe_w["w"] = ((torch.randn((E, 2 * I, H), generator=g) * 0.02).to(torch.bfloat16),
+                              (torch.randn((E, H, I), generator=g) * 0.02).to(torch.bfloat16))
+        w1, w2 = cpu_moe_w["w"]
+        x = torch.randn((T, H), generator=g).to(torch.bfloat16)
+        logits = torch.randn((T, E), generator=g).to(torch.bfloat16)
+        dt_s, reps = cpu_time(lambda: omoe.torch_path_fused_moe(x, w1, w2, logits, K, renormalize=True),
+                              budget_s=1.0, min_reps=2, max_reps=20)
+        sample_bytes = E * 3 * I * H * 2 + 2 * T * H * 2 + T * E * 2
+        return dict(value=round(sample_bytes / dt_s / 1e9, 3), unit="GB/s", us_scaled_to_full=round(dt_s * 1e6 * slab, 1),
+                    cores=cores, kind="port",
+                    sample="dense torch MoE in bf16 (softmax, top-2, renormalised, all 8 experts on every token) with "
+                           "H=4096 and 1/%d of the intermediate size (I=%d), T=%d, %d reps, %.1f ms each; host has %d "
+                           "logical CPUs" % (slab, I, T, reps, dt_s * 1e3, host_cpus))
+
+    # ------------------------------------------------------------------ GPU cases
+    def gemv_case(name, n, k, kind, steps, warmup, yardstick=False, cpu_rows=2048):
         xk = 1 if kind == 2 else kind
-        A = weights(n, k, kind, copies_for(n * k * (1 if kind == 2 else 2)))
+        wbytes = n * k * (1 if kind == 2 else 2)
+        A = weights(n, k, kind, copies_for(wbytes))
         x = torch.randn((1, k), generator=gen, device=dev).to(DT[xk])
         y = torch.empty((1, n), dtype=DT[xk], device=dev)
         scale = torch.ones(((n + 127) // 128, (k + 127) // 128), dtype=torch.float32, device=dev) if kind == 2 else None
@@ -126,22 +243,22 @@ def main():
                                                  0 if scale is None else scale.data_ptr(), block, kid, p1, p2, st),
                            "gemv")
             return call
-        us, wall = run_graph([mk(a) for a in A], steps, warmup)
-        algo = n * k * (1 if kind == 2 else 2) + (scale.numel() * 4 if scale is not None else 0) + k * 2 + n * 2
-        return dict(name=name, us=us, bytes=algo, gbps=algo / us / 1e3, frac=algo / us / 1e3 / HBM_PEAK_GBPS,
-                    params=[block, kid, p1, p2], copies=len(A), wall=wall)
+        t = run_graph([mk(a) for a in A], steps, warmup)
+        algo = wbytes + (scale.numel() * 4 if scale is not None else 0) + k * 2 + n * 2
+        extra = dict(params=[block, kid, p1, p2], copies=len(A))
+        del A
+        if yardstick:
+            extra["read_only_us"] = read_only_us(wbytes, min(steps, 60))
+        extra["cpu_baseline"] = cpu_linear(n, k, 1, kind, cpu_rows)
+        return finish(name, t, algo, **extra)
 
-    def gemm_case(name, n, k, kind, m, steps, warmup, native=False, copies=None):
+    def gemm_case(name, n, k, kind, m, steps, warmup, native=False, copies=None, cpu_rows=2048, cpu=True):
         xk = 1 if kind == 2 else kind
         A = weights(n, k, kind, copies or copies_for(n * k * (1 if kind == 2 else 2)))
         b = torch.randn((m, k), generator=gen, device=dev).to(DT[xk])
         scale = torch.ones((n // 128, k // 128), dtype=torch.float32, device=dev) if kind == 2 else None
         table = "layoutA_soft_fp8_gemm" if kind == 2 else ("layout_gemm" if native else "layoutA_gemm")
         kid, p1, p2, p3 = mlk.ops._gemm_guard(arg_selector.selector(table).get_args((n, m, k)), n)
-        ws_ptr, ws_len = 0, 0
-        if p3 > 1:
-            ws = mlk.ops._workspace(dev, lib.mlk_gemm_workspace_bytes(m, n, p1, p3), lib.mlk_gemm_counter_bytes())
-            ws_ptr, ws_len = ws.data_ptr(), ws.numel()
         if native:
             b_in = mlk.layoutB(b)
             c = torch.empty((n // 32, m // 16, 4, 16, 8), dtype=DT[xk], device=dev)
@@ -153,6 +270,10 @@ def main():
         def mk(a):
             def call():
                 st = torch.cuda.current_stream().cuda_stream
+                ws_ptr, ws_len = 0, 0
+                if p3 > 1:      # per-stream scratch of the K split (allocated by the warm-up calls, before the capture)
+                    ws = mlk.ops._workspace(dev, lib.mlk_gemm_workspace_bytes(m, n, p1, p3), lib.mlk_gemm_counter_bytes(), st)
+                    ws_ptr, ws_len = ws.data_ptr(), ws.numel()
                 _lib.check(lib.mlk_gemm_layout_a(a.data_ptr(), b_in.data_ptr(), c.data_ptr(), m, n, k, kind, xk,
                                                  1 if native else 0, 1 if native else 0, 1.0, 0,
                                                  0 if scale is None else scale.data_ptr(), kid, p1, p2, p3, ws_ptr, ws_len,
@@ -161,20 +282,31 @@ def main():
                 if native:
                     _lib.check(lib.mlk_re_layout_c(c.data_ptr(), c_rm.data_ptr(), m, n, st), "reLayoutC")
             return call
-        us, wall = run_graph([mk(a) for a in A], steps, warmup)
+        t = run_graph([mk(a) for a in A], steps, warmup)
         algo = n * k * (1 if kind == 2 else 2) + (scale.numel() * 4 if scale is not None else 0) + m * k * 2 + m * n * 2
         if native:
             algo += 2 * m * n * 2
-        return dict(name=name, us=us, bytes=algo, gbps=algo / us / 1e3, frac=algo / us / 1e3 / HBM_PEAK_GBPS,
-                    params=[kid, p1, p2, p3], copies=len(A), wall=wall)
+        row = finish(name, t, algo, params=[kid, p1, p2, p3], copies=len(A))
+        if cpu:
+            row["cpu_baseline"] = cpu_linear(n, k, m, kind, cpu_rows, native=native)
+        return row
 
     def panel_case(name, n, k, kind, m, steps):
-        """Prefill-sized token counts: bound by the matrix cores (or by the weight stream up to ~300 tokens)."""
-        row = gemm_case(name, n, k, kind, m, steps, 3, copies=2)
+        """Prefill-sized token counts: bound by the matrix cores (or by the weight stream up to ~300 tokens).
+        The vendor BLAS on an un-packed 16-bit copy of the same shape is timed beside it."""
+        row = gemm_case(name, n, k, kind, m, steps, 3, copies=2, cpu=False)
         flops = 2.0 * m * n * k
         row["tflops"] = flops / row["us"] / 1e6
         row["mfma_frac"] = row["tflops"] / MFMA_PEAK_TFLOPS
         row["bound"] = "mfma" if flops / (MFMA_PEAK_TFLOPS * 1e6) > row["bytes"] / (HBM_PEAK_GBPS * 1e3) else "hbm"
+        dt = torch.bfloat16 if kind == 2 else DT[kind]
+        W = [(torch.randn((n, k), generator=gen, device=dev) * 0.02).to(dt) for _ in range(2)]
+        b = torch.randn((m, k), generator=gen, device=dev).to(dt)
+        out = torch.empty((m, n), dtype=dt, device=dev)
+        t = run_graph([(lambda w=w: torch.matmul(b, w.t(), out=out)) for w in W], steps, 3, reps=3)
+        row["blas_us"] = t["us_median"]
+        row["blas_tflops"] = flops / t["us_median"] / 1e6
+        row["blas_note"] = "torch.matmul (vendor BLAS) on un-packed %s weights of the same shape" % str(dt).replace("torch.", "")
         return row
 
     moe_w = {}
@@ -207,15 +339,20 @@ def main():
         y = call()
         ids = torch.topk(torch.softmax(logits.float(), dim=-1), K, dim=-1).indices
         e_act = int(torch.unique(ids).numel())
-        us, wall = run_graph([call], steps, warmup)
+        t = run_graph([call], steps, warmup)
         wbytes = 1 if fp8 else 2
         algo = e_act * 3 * I * H * wbytes + 2 * T * H * 2 + T * E * 2
         if fp8:
             algo += e_act * 3 * (I // 128) * (H // 128) * 4
         del y
-        return dict(name=name, us=us, bytes=algo, gbps=algo / us / 1e3, frac=algo / us / 1e3 / HBM_PEAK_GBPS,
-                    active_experts=e_act, roofline_us=algo / HBM_PEAK_GBPS / 1e3,
-                    ratio_to_roofline=us / (algo / HBM_PEAK_GBPS / 1e3), wall=wall)
+        roof = algo / HBM_PEAK_GBPS / 1e3
+        row = finish(name, t, algo, active_experts=e_act, roofline_us=roof, ratio_to_roofline=t["us"] / roof)
+        base = cpu_moe(T)
+        if base is not None and fp8:
+            base = dict(base, sample=base["sample"] + "; the reference's CPU path for soft-FP8 weights is the same loop "
+                                                      "on weights widened to bf16 beforehand")
+        row["cpu_baseline"] = base
+        return row
 
     def moe_next_case(name, T, steps, warmup):
         """The routing configuration the reference's own router is written for (256 experts in 8 groups, 4 groups
@@ -243,12 +380,51 @@ def main():
         wts = torch.empty((T, K), dtype=torch.bfloat16, device=dev)
         mlk.fused_routing_gate(logits, 1, T, H, 8, 4, ids, wts, K, bias)
         e_act = int(torch.unique(ids).numel())
-        us, wall = run_graph([call], steps, warmup)
+        t = run_graph([call], steps, warmup)
         algo = e_act * 3 * I * H * 2 + 2 * T * H * 2 + T * E * 2
         del y
-        return dict(name=name, us=us, bytes=algo, gbps=algo / us / 1e3, frac=algo / us / 1e3 / HBM_PEAK_GBPS,
-                    active_experts=e_act, roofline_us=algo / HBM_PEAK_GBPS / 1e3,
-                    ratio_to_roofline=us / (algo / HBM_PEAK_GBPS / 1e3), wall=wall)
+        roof = algo / HBM_PEAK_GBPS / 1e3
+        return finish(name, t, algo, active_experts=e_act, roofline_us=roof, ratio_to_roofline=t["us"] / roof)
+
+    def relayout_case(name, which, steps):
+        """The relayout / repack kernels: read + write of the tensor."""
+        st_of = lambda: torch.cuda.current_stream().cuda_stream     # noqa: E731
+        if which == "fp8_weight_repack":
+            n, k = 28672, 8192
+            src = [torch.randint(0, 255, (n, k), dtype=torch.uint8, device=dev) for _ in range(2)]
+            dst = torch.empty_like(src[0])
+            calls = [(lambda a=a: _lib.check(lib.mlk_fp8_weight_repack(a.data_ptr(), dst.data_ptr(), a.numel(), st_of()),
+                                             "repack")) for a in src]
+            algo = 2 * n * k
+        elif which == "layoutB":
+            m, k = 32, 8192
+            src = [torch.randn((m, k), generator=gen, device=dev).to(torch.bfloat16) for _ in range(4)]
+            dst = torch.empty((k // 32, m // 16, 4, 16, 8), dtype=torch.bfloat16, device=dev)
+            calls = [(lambda a=a: _lib.check(lib.mlk_layout_b(a.data_ptr(), dst.data_ptr(), m, k, st_of()), "layoutB"))
+                     for a in src]
+            algo = 2 * m * k * 2
+        else:
+            m, n = 32, 8192
+            src = [torch.randn((n // 32, m // 16, 4, 16, 8), generator=gen, device=dev).to(torch.bfloat16) for _ in range(4)]
+            dst = torch.empty((m, n), dtype=torch.bfloat16, device=dev)
+            calls = [(lambda a=a: _lib.check(lib.mlk_re_layout_c(a.data_ptr(), dst.data_ptr(), m, n, st_of()), "reLayoutC"))
+                     for a in src]
+            algo = 2 * m * n * 2
+        t = run_graph(calls, steps, 3)
+        return finish(name, t, algo)
+
+    def pack_case(name, e, n, k, steps):
+        """The device step of the checkpoint converter: row-major expert matrices -> layout-A (read + write)."""
+        src = [(torch.randn((e, n, k), generator=gen, device=dev) * 0.02).to(torch.bfloat16) for _ in range(2)]
+        dst = torch.empty((e, n // 16, k // 8, 16, 8), dtype=torch.bfloat16, device=dev)
+
+        def mk(a):
+            def call():
+                _lib.check(lib.mlk_pack_layout_a(a.data_ptr(), dst.data_ptr(), e, n, k, 2,
+                                                 torch.cuda.current_stream().cuda_stream), "pack_layout_a")
+            return call
+        t = run_graph([mk(a) for a in src], steps, 3)
+        return finish(name, t, 2 * e * n * k * 2)
 
     if args.calibrate_copy:
         src = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device=dev)
@@ -269,59 +445,48 @@ def main():
                     _lib.check(lib.mlk_stream_read(b.data_ptr(), nbytes, block, wgs, 0,
                                                    torch.cuda.current_stream().cuda_stream), "stream_read")
                 return call
-            us, _ = run_graph([mk(b) for b in bufs], steps, 5)
-            best = max(best, nbytes / us / 1e3)
+            t = run_graph([mk(b) for b in bufs], steps, 5, reps=3)
+            best = max(best, nbytes / t["us_median"] / 1e3)
         return best
-
-    def pack_case(name, e, n, k, steps):
-        """The device step of the checkpoint converter: row-major expert matrices -> layout-A (read + write)."""
-        src = [(torch.randn((e, n, k), generator=gen, device=dev) * 0.02).to(torch.bfloat16) for _ in range(2)]
-        dst = torch.empty((e, n // 16, k // 8, 16, 8), dtype=torch.bfloat16, device=dev)
-
-        def mk(a):
-            def call():
-                _lib.check(lib.mlk_pack_layout_a(a.data_ptr(), dst.data_ptr(), e, n, k, 2,
-                                                 torch.cuda.current_stream().cuda_stream), "pack_layout_a")
-            return call
-        us, wall = run_graph([mk(a) for a in src], steps, 3)
-        algo = 2 * e * n * k * 2
-        return dict(name=name, us=us, bytes=algo, gbps=algo / us / 1e3, frac=algo / us / 1e3 / HBM_PEAK_GBPS, wall=wall)
 
     # ------------------------------------------------------------ headline
     N, K_, M = 11008, 4096, 16
-    head = gemm_case("C2 fp16 gemm_layoutA 11008x4096 M=16", N, K_, 0, M, args.steps, args.warmup)
+    HEAD = "C2 fp16 gemm_layoutA 11008x4096 M=16"
+    head = gemm_case(HEAD, N, K_, 0, M, args.steps, args.warmup)
     per_config = []
 
     def add(case, name, *a, **kw):
         """Run one per-configuration case unless --case asks for others only."""
-        if args.case is None or args.case in name:
+        if args.case is None or any(part and part in name for part in args.case.split(",")):
             per_config.append(case(name, *a, **kw))
     ceiling = None
     resident = None
+    same_size = None
     if not args.quick:
         one = gemm_case("headline workload, one weight copy (stays in the 256 MiB Infinity Cache)", N, K_, 0, M, args.steps,
-                        args.warmup, copies=1)
+                        args.warmup, copies=1, cpu=False)
         resident = {"us_per_call": round(one["us"], 3), "gbps": round(one["gbps"], 1),
                     "what": "same kernel and launch parameters on a single 86 MiB weight copy: the stream comes from "
                             "the Infinity Cache, not HBM; reported for information, never the headline"}
         ceiling = round(read_ceiling(40), 1)
         # the same yardstick at the headline's size: one launch that only reads as many bytes as the weights hold
-        wbytes = N * K_ * 2
-        same_size = wbytes / read_ceiling(min(args.steps, 100), wbytes - wbytes % 4096, copies_for(wbytes),
-                                          ((512, 1024), (1024, 512), (256, 2048), (512, 512))) / 1e3
+        same_size = read_only_us(N * K_ * 2, min(args.steps, 100))
         short = max(20, min(args.steps, 100))
-        add(gemv_case, "C1 bf16 gemv 4096x4096", 4096, 4096, 1, short, 10)
+        add(gemv_case, "C1 bf16 gemv 4096x4096", 4096, 4096, 1, short, 10, yardstick=True, cpu_rows=4096)
         for m in (1, 8, 32, 64):
             add(gemm_case, "C2 fp16 gemm_layoutA 11008x4096 M=%d" % m, N, K_, 0, m, short, 10)
         add(gemv_case, "C2 fp16 gemv 11008x4096", N, K_, 0, short, 10)
-        add(gemv_case, "C3 soft-fp8 gemv 28672x8192", 28672, 8192, 2, short, 10)
+        add(gemv_case, "C3 soft-fp8 gemv 28672x8192", 28672, 8192, 2, short, 10, yardstick=True, cpu_rows=1024)
         for m in (4, 16):
-            add(gemm_case, "C3 soft-fp8 gemm_layoutA 28672x8192 M=%d" % m, 28672, 8192, 2, m, short, 10)
-        add(gemm_case, "C4 bf16 gemm_layoutABC+reLayoutC 8192x8192 M=32", 8192, 8192, 1, 32, short, 10,
-                                    native=True)
+            add(gemm_case, "C3 soft-fp8 gemm_layoutA 28672x8192 M=%d" % m, 28672, 8192, 2, m, short, 10, cpu_rows=1024)
+        add(gemm_case, "C4 bf16 gemm_layoutABC+reLayoutC 8192x8192 M=32", 8192, 8192, 1, 32, short, 10, native=True,
+            cpu_rows=1024)
+        add(relayout_case, "C4 layoutB bf16 [32, 8192]", "layoutB", short)
+        add(relayout_case, "C4 reLayoutC bf16 [32, 8192]", "reLayoutC", short)
+        add(relayout_case, "C3 fp8_weight_repack 28672x8192", "fp8_weight_repack", 10)
         for T in (1, 16, 64, 256):
             add(moe_case, "C5 bf16 fused_moe T=%d" % T, T, False, 20, 5)
-        for T in (1, 16):
+        for T in (1, 16, 64, 256):
             add(moe_case, "C5 soft-fp8 fused_moe T=%d" % T, T, True, 20, 5)
         for T in (1, 16):
             add(moe_next_case, "next: grouped-routing MoE E=256 top-8 H=7168 I=2048 bf16 T=%d" % T, T, 20, 5)
@@ -336,38 +501,10 @@ def main():
         torch.cuda.empty_cache()
         for row in per_config:
             row.pop("wall", None)
-            for key in ("us", "gbps", "frac", "roofline_us", "ratio_to_roofline", "tflops", "mfma_frac"):
-                if key in row:
+            for key in ("us", "us_median", "us_min", "gbps", "frac", "roofline_us", "ratio_to_roofline", "tflops",
+                        "mfma_frac", "read_only_us", "blas_us", "blas_tflops", "traffic_over_algorithmic"):
+                if row.get(key) is not None:
                     row[key] = round(row[key], 4)
-
-    # -------------------------------------------------------- CPU baseline
-    cpu = None
-    if not args.no_cpu:
-        from oracle import gemm as ogemm
-        rows = 2048                                    # bounded sample: the first 2048 of 11008 weight rows
-        g = torch.Generator().manual_seed(2025)
-        w = (torch.randn((rows, K_), generator=g) * 0.02).to(torch.float16)
-        b = torch.randn((M, K_), generator=g).to(torch.float16)
-        for _ in range(2):
-            ogemm.torch_path_linear(w, b)
-        reps, t0 = 0, time.perf_counter()
-        while reps < 5 or (time.perf_counter() - t0 < 5.0 and reps < 200):
-            ogemm.torch_path_linear(w, b)
-            reps += 1
-        dt = (time.perf_counter() - t0) / reps
-        sample_bytes = rows * K_ * 2 + M * K_ * 2 + M * rows * 2
-        cpu = dict(value=round(sample_bytes / dt / 1e9, 3), unit="GB/s", cores=torch.get_num_threads(),
-                   kind="port",
-                   sample="torch linear in fp16 on the first %d of %d un-packed weight rows, M=%d, %d reps, %.3f ms each; "
-                          "host has %d logical CPUs" % (rows, N, M, reps, dt * 1e3, os.cpu_count() or 0))
-
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "hbm_traffic.json")
-    if os.path.exists(tpath):
-        try:
-            traffic = json.load(open(tpath)).get("C2 fp16 gemm_layoutA 11008x4096 M=16")
-        except (OSError, ValueError):
-            traffic = None
 
     line = {
         "metric": "achieved GB/s of algorithmic bytes per call (us/call and % of HBM peak alongside)",
@@ -378,6 +515,8 @@ def main():
         "warmup": args.warmup,
         "ms_per_step": round(head["wall"] * 1e3 / args.steps, 6),
         "us_per_call": round(head["us"], 3),
+        "us_per_call_median_of_%d_replays" % TIMED_REPLAYS: round(head["us_median"], 3),
+        "us_per_call_min_of_%d_replays" % TIMED_REPLAYS: round(head["us_min"], 3),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -388,13 +527,13 @@ def main():
                    "untimed_graph_replays_before_timing": settle_replays(args.steps), "launch_params": head["params"],
                    "algorithmic_bytes": head["bytes"]},
         "roofline": {"bound": "hbm", "achieved": round(head["gbps"], 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(head["frac"], 4), "traffic": traffic},
+                     "frac": round(head["frac"], 4), "traffic": traffic_table.get(HEAD)},
         "hbm_read_ceiling": None if ceiling is None else {
             "value": ceiling, "unit": "GB/s",
             "what": "pure streaming read (mlk_stream_read, 256 MiB x 4 rotating buffers) measured in this run",
             "us_for_one_launch_reading_the_headline_weights": round(same_size, 3)},
         "infinity_cache_resident": resident,
-        "cpu_baseline": cpu,
+        "cpu_baseline": head.get("cpu_baseline"),
         "per_config": per_config,
     }
     print(json.dumps(line))

@@ -63,6 +63,11 @@ const char *mlk_last_error(void);
  *         soft-FP8 weights, 4 otherwise)
  *   id 7  decode MoE (2..16 tokens), down kernel: row groups per wave = K slices across
  *         workgroups, 1, 2 or 4 (default 0 = 4 for soft-FP8 weights, 1 otherwise)
+ *   id 8  fused MoE above 16 tokens: upper limit of the token blocks (of 16) that share one pass over an
+ *         expert's weights, 1..8 (default 0 = sized from the expected load of an expert)
+ *   id 9  fused MoE, soft-FP8 weights, more than 64 tokens per pass over an expert: 1 keeps the row-shared
+ *         kernels instead of the panel kernels (default 0)
+ * The MoE scan script (kernel_args_scan/moe_scan.py) sweeps ids 2..5, 7 and 8.
  * No counterpart in the reference. */
 void mlk_set_tunable(int id, int value);
 /* Experiment switches of the fused MoE: bit 0 set (default) = use the row-shared kernels for more
@@ -113,10 +118,18 @@ int mlk_stream_read(const void *src, int64_t nbytes, int block_dim_x, int workgr
  * N % 16 == 0, K % 32 == 0 (K % 64 == 0 for fp8).
  * Launch parameters (what the reference's csv rows select):
  *   block_dim_x  threads per workgroup, 64..1024, multiple of 64
- *   kernel_id    1 = streaming kernel (the only one)
- *   p1           row groups (of 16 rows) per workgroup: >= 1 and divides both N/16 and
- *                block_dim_x/64; the block_dim_x/64/p1 waves of a row group split K
- *   p2           16-byte loads kept in flight per wave: 1, 2, 4, 6 or 8
+ *   kernel_id    1 = streaming kernel, a workgroup per p1 row groups
+ *                2 = the same stream, but the grid is p1 workgroups per CU and each workgroup walks a
+ *                    contiguous range of row groups (dealt out evenly) in one uninterrupted stream per wave,
+ *                    with the whole activation vector staged in LDS once (falls back to kernel 1 when
+ *                    M * K * 2 bytes plus the partial sums exceed 64 KiB of LDS)
+ *                3 = kernel 2 with the products on the matrix cores (soft-FP8 weights only; 16-bit weights
+ *                    run kernel 2): two v_mfma_f32_16x16x32_bf16 per 1 KiB tile take the even and the odd
+ *                    rows, the widening stays on the vector ALU
+ *   p1           kernel 1: row groups (of 16 rows) per workgroup: >= 1 and divides both N/16 and
+ *                block_dim_x/64; the block_dim_x/64/p1 waves of a row group split K.
+ *                kernels 2, 3: workgroups per CU, 1..16
+ *   p2           16-byte loads kept in flight per wave: 1, 2, 4, 6 or 8 (kernels 2, 3: not 1)
  */
 int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k, int a_kind, int x_kind,
                       float alpha, const void *bias, const float *scale, int block_dim_x, int kernel_id, int p1,

@@ -14,8 +14,11 @@ What the columns select on gfx950 (the rows are produced by the scripts in
 
   GeMV tables   m,k -> BLOCK_DIM_X, KernelId, KernelParam1, KernelParam2
                 BLOCK_DIM_X  threads per workgroup (64..1024)
-                KernelId     1 = streaming GeMV
-                KernelParam1 row groups (16 rows) per workgroup
+                KernelId     1 = streaming GeMV, one workgroup per KernelParam1 row groups
+                             2 = the same stream from KernelParam1 workgroups per CU, each walking a
+                                 contiguous range of row groups in one uninterrupted stream per wave
+                             3 = kernel 2 with the products of soft-FP8 weights on the matrix cores
+                KernelParam1 row groups (16 rows) per workgroup (kernel 1) / workgroups per CU (2, 3)
                 KernelParam2 16-byte loads kept in flight per wave
   GEMM tables   m,n,k -> kernelId, kernelParam1, kernelParam2, kernelParam3
                 kernelId     1 = wave-tiled MFMA kernel (waves of a workgroup split K)
@@ -184,9 +187,13 @@ def gemv_guard(args, n, k):
     that asks for more row groups per workgroup than divide N/16, or more than
     the wave count allows, is replaced by the plain configuration."""
     block, kid, p1, p2 = args
-    if kid != 1 or p1 < 1 or (n // 16) % p1 != 0 or (block // 64) % p1 != 0 or block % 64 or not 64 <= block <= 1024:
+    if block % 64 or not 64 <= block <= 1024 or p2 not in (1, 2, 4, 6, 8):
         return (256, 1, 1, 4)
-    return args
+    if kid == 1 and p1 >= 1 and (n // 16) % p1 == 0 and (block // 64) % p1 == 0:
+        return args
+    if kid in (2, 3) and 1 <= p1 <= 16 and p2 != 1:       # p1 = workgroups per CU
+        return args
+    return (256, 1, 1, 4)
 
 
 def parse_table_text(text, key_cells):

@@ -23,7 +23,7 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 // Experiment switches set through mlk_set_tunable().
-extern int g_tunable[8];
+extern int g_tunable[16];
 
 // Record an error message for mlk_last_error() and return the code.
 int fail(int code, const char *msg);

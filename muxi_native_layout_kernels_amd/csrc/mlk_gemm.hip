@@ -47,8 +47,8 @@ static int static_scratch(void **out, hipStream_t s) {
 
 // Experiment switches (mlk_set_tunable): [0] rotate the k-tile order per row tile,
 // [1] stage row-major activations through LDS, [2]..[5] and [7] shape the fused MoE kernels
-// (listed with the declaration of mlk_set_tunable); 0 means automatic for [5] and [7].
-int g_tunable[8] = {1, 1, 1, 8, 16, 0, 0, 0};
+// (listed with the declaration of mlk_set_tunable); 0 means automatic for [5], [7] and [8].
+int g_tunable[16] = {1, 1, 1, 8, 16, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
 extern template int launch_modes<F16, false>(const GemmArgs &, int, int, int, int, int, hipStream_t);
 extern template int launch_modes<BF16, false>(const GemmArgs &, int, int, int, int, int, hipStream_t);
@@ -65,7 +65,7 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
 using namespace mlk;
 
 extern "C" void mlk_set_tunable(int id, int value) {
-    if (id >= 0 && id < 8) g_tunable[id] = value;
+    if (id >= 0 && id < 16) g_tunable[id] = value;
 }
 
 extern "C" size_t mlk_gemm_counter_bytes(void) { return kCounterBytes; }

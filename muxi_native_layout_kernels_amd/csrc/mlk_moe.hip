@@ -25,7 +25,7 @@
 // read once) stays in L2 / Infinity Cache for decode-sized T.
 #include <math.h>
 
-#include "mlk_tile.cuh"
+#include "mlk_moe_args.cuh"
 
 namespace mlk {
 
@@ -45,7 +45,8 @@ static inline int moe_blocks_per_task(int tokens, int topk, int experts) {
     int expect = (int)(mean + 3.0 * sqrt(mean)) + 1;
     if (expect > tokens) expect = tokens;
     int cb = (expect + 15) / 16;
-    const int cap = moe_tile_path() ? 8 : 4;
+    int cap = moe_tile_path() ? 8 : 4;
+    if (g_tunable[8] > 0 && g_tunable[8] < cap) cap = g_tunable[8];      // experiment switch: fewer blocks per task
     if (cb > cap) cb = cap;
     if (cb == 5) cb = 6;
     if (cb == 7) cb = 8;
@@ -254,9 +255,6 @@ __global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__
 }
 
 // ------------------------------------------------------------------- align
-struct MoeTask {
-    int expert, block0, nblocks, pad;
-};
 
 __global__ void __launch_bounds__(1024) moe_align_kernel(const int32_t *__restrict__ topk_ids, int n_pairs, int E,
                                                          const int32_t *__restrict__ experts_map,
@@ -366,25 +364,6 @@ __device__ __forceinline__ size_t hbuf_offset(int n, int block, int token, int S
     return ((((size_t)(n >> 5) * SB + block) * 16 + token) * 4 + ((n & 31) >> 3)) * 8 + (n & 7);
 }
 
-struct MoeArgs {
-    const uint8_t *W1;        // [E][2I][H] layout-A slabs
-    const uint8_t *W2;        // [E][H][I]
-    const float *S1;          // [E][2I/128][H/128] or null
-    const float *S2;          // [E][H/128][I/128] or null
-    const uint16_t *X;        // [T][H]
-    uint16_t *Y;              // [T][H]
-    uint16_t *Hbuf;           // layout-B [I/32][SB][4][16][8]
-    const uint16_t *wts;      // [T*K]
-    const int32_t *sorted;    // [T*K + E*15]
-    const MoeTask *tasks;
-    const int32_t *n_tasks;
-    const int32_t *topk_ids;  // [T*K], read by the decode variants that align in-kernel
-    const int32_t *experts_map;
-    int T, K, H, I, SB, n_pairs, WK, E;
-    float *part;              // down projection with K slices: fp32 partial output tiles [slice][workgroup][T][16R]
-    int32_t *counters;        // arrival counters, one per down workgroup column (zeroed by the gate/up kernel)
-    int n_counters;
-};
 
 // Decode-sized batches (T*K <= 64 pairs): every workgroup rebuilds the tiny alignment itself
 // from the routing table instead of waiting for a separate alignment launch.  One wave walks
@@ -1288,8 +1267,25 @@ static int launch_moe_cb(const MoeArgs &a, int cb, int max_tasks, bool inline_al
     }
 }
 
+extern template int launch_moe_panel<BF16, true>(const MoeArgs &, int, int, float *, int, hipStream_t);
+
+// K slices of the panel down projection: its grid is (H / 256 row tiles, tasks, slices); slice K while the grid
+// holds fewer than one and a half workgroups per CU and a slice keeps at least four 128-wide k windows.
+static int moe_panel_down_slices(int hidden, int inter, int max_tasks) {
+    const int row_tiles = hidden / 256, windows = inter / 128, cus = device_cus();
+    int skd = 1;
+    while (skd < kMoeMaxKSlices && row_tiles * max_tasks * skd * 2 < cus * 3 && windows / (skd * 2) >= 4) skd *= 2;
+    return skd;
+}
+// blocks of 32 tokens in a panel for tasks of up to cb blocks of 16
+static int moe_panel_tb32(int cb) { return (cb + 1) / 2 > 4 ? 4 : (cb + 1) / 2; }
+// The panel kernels take soft-FP8 weights from five token blocks per task on (more than 64 tokens per pass over an
+// expert: the matrix cores, not the weight stream, set the pace there) when the output rows tile in 256.
+// Experiment switch 9: 1 keeps the row-shared kernels.
+static bool moe_panel_path(int cb, int hidden, bool fp8) { return fp8 && cb >= 5 && hidden % 256 == 0 && g_tunable[9] != 1; }
+
 // How one pass of up to kMoeChunk tokens is run.  The launch code below and mlk_moe_plan() both read it.
-enum { kMoePathGemv1 = 0, kMoePathDecodeInline = 1, kMoePathDecode = 2, kMoePathTile = 3 };
+enum { kMoePathGemv1 = 0, kMoePathDecodeInline = 1, kMoePathDecode = 2, kMoePathTile = 3, kMoePathPanel = 4 };
 struct MoePlan {
     int path;         // kMoePath*
     int cb;           // token blocks per task
@@ -1313,6 +1309,12 @@ static MoePlan moe_plan(int tc, int n_experts, int topk, int hidden, int inter, 
     }
     const bool inline_align = tc <= 16 && n_pairs <= kDecodePairs;
     if (inline_align) pl.cb = 1;
+    if (!inline_align && moe_tile_path() && moe_panel_path(pl.cb, hidden, fp8)) {
+        pl.path = kMoePathPanel;
+        pl.down_r = 4;
+        pl.down_slices = moe_panel_down_slices(hidden, inter, pl.max_tasks);
+        return pl;
+    }
     if (!inline_align && pl.cb >= 2 && (moe_tile_path() || pl.cb > 4)) {
         pl.path = kMoePathTile;
         pl.down_r = moe_tile_down_rows(pl.cb, hidden);
@@ -1515,6 +1517,15 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
         a.counters = ws.counters;
         a.n_counters = hidden / 16;
         int rc;
+        if (pl.path == kMoePathPanel) {
+            const int tb32 = moe_panel_tb32(cb), skd = pl.down_slices;
+            const dim3 cgrid(tc, (hidden + 1023) / 1024);
+            rc = launch_moe_panel<BF16, true>(a, tb32, max_tasks, ws.obuf, skd, s);
+            if (rc != MLK_OK) return rc;
+            moe_combine_kernel<BF16><<<cgrid, 256, 0, s>>>(ws.obuf, a.Y, a.topk_ids, a.experts_map, topk, hidden, n_experts, skd);
+            MLK_LAUNCH_CHECK();
+            continue;
+        }
         if (fp8) rc = launch_moe_cb<BF16, true>(a, cb, max_tasks, inline_align, ws.obuf, s);
         else if (x_kind == MLK_F16) rc = launch_moe_cb<F16, false>(a, cb, max_tasks, inline_align, ws.obuf, s);
         else rc = launch_moe_cb<BF16, false>(a, cb, max_tasks, inline_align, ws.obuf, s);

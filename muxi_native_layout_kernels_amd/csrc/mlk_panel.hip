@@ -27,19 +27,9 @@
 // picks the XCD), so the weights of a row tile are read from HBM once and served to the other token
 // tiles by that XCD's L2.  K slices fold like in the row-shared kernel: fp32 partials with
 // agent-scope stores, the last workgroup to arrive adds them in slice order.
-#include <type_traits>
-
-#include "mlk_tile.cuh"
+#include "mlk_panel_loop.cuh"
 
 namespace mlk {
-
-// Two panel shapes: TB = 4 blocks of 32 tokens (128 tokens, k windows of 128) and TB = 8 (256 tokens, k windows
-// of 64).  What a CU can pull through its memory path bounds the kernel once the matrix cores are fed, and a
-// 256 x 256 panel moves a third fewer operand bytes per flop than a 256 x 128 one.
-constexpr int kPanelRowsPerWg = kTileWaves * 4 * 16;         // 256 rows: two pairs of row groups per wave (128 with one pair)
-__host__ __device__ constexpr int panel_kw(int tb) { return tb == 4 ? 4 : 2; }                 // k tiles per window
-__host__ __device__ constexpr int panel_tile_stride(int tb) { return tb * 4 * 33 + 4; }         // granules between k tiles
-__host__ __device__ constexpr int panel_win(int tb) { return panel_kw(tb) * panel_tile_stride(tb); }
 
 struct PanelArgs {
     const uint8_t *A;
@@ -55,22 +45,11 @@ struct PanelArgs {
     float alpha;
 };
 
-// Two vertically adjacent layout-A fragments -> the 32x32x16 operands of k octets {0, 1} (in x) and {2, 3} (in y).
-__device__ __forceinline__ void pair_to_rows32(u32x4 &x, u32x4 &y) {
-#pragma unroll
-    for (int d = 0; d < 4; ++d) {
-        auto s16 = __builtin_amdgcn_permlane16_swap(x[d], y[d], false, false);
-        auto s32 = __builtin_amdgcn_permlane32_swap(s16[0], s16[1], false, false);
-        x[d] = s32[0];
-        y[d] = s32[1];
-    }
-}
-
 template <class T, bool FP8, int TB, int PR>
 __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     extern __shared__ u32x4 win[];
     __shared__ int s_last;
-    constexpr int R = 2 * PR, KW = panel_kw(TB), WG = panel_win(TB), TS = panel_tile_stride(TB);   // PR pairs of row groups per wave
+    constexpr int R = 2 * PR, KW = panel_kw(TB);               // PR pairs of row groups per wave
     constexpr int WBYTES = FP8 ? 1 : 2;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -98,7 +77,6 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
         const int rg = min(rg0 + r, groups - 1);              // rows past N are computed on a copy and never stored
         abase[r] = p.A + (size_t)rg * p.K * 16 * WBYTES;
     }
-    const uint32_t lane_off = lane * (FP8 ? 8 : 16);
     ScaleRow srow;
     if (FP8) srow = load_scale_row(p.scale ? p.scale + (size_t)(min(rg0, groups - 1) >> 3) * scale_cols : nullptr, scale_cols, lane);
 
@@ -112,10 +90,6 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
         const int tok = min(tok0 + trow + RP * i, p.M - 1);
         boff[i] = (uint32_t)tok * (uint32_t)p.K + colg * 8;
     }
-    const int st_idx = (colg >> 2) * TS + (colg & 3) * 33 + trow;             // + st_off(i)
-    auto st_off = [](int i) { return ((RP * i) / 32) * 4 * 33 + (RP * i) % 32; };
-    const int ld_idx = (lane >> 5) * 33 + (lane & 31);                        // + t * TS + (tb * 4 + 2 s) * 33
-
     f32x16 acc[PR][TB];
 #pragma unroll
     for (int pr = 0; pr < PR; ++pr)
@@ -124,138 +98,10 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[pr][tb][e] = 0.f;
 
-    // Pipeline of one window j (128 k; weight slot j & 1, LDS buffer j % 3) in eight half steps of eight
-    // MFMAs (16 k x four token blocks x two row pairs).  While a half step multiplies out of one set of
-    // fragment registers the LDS reads of the next half step land in the other set.  Everything that
-    // comes from memory is requested well before it is used: the weights of tile t of window j + 2
-    // once tile t of window j has been multiplied (same registers), the activations of window
-    // j + 2 at the start of window j; they are written to LDS in the middle of window j + 1 and
-    // published by the single barrier there, so that the reads of the first half step of window
-    // j + 2 can go out during the last half step of window j + 1.  With three LDS buffers that one
-    // barrier per window is enough: the buffer written in the middle of window j was last read in
-    // window j - 2, which every wave has left before it reaches the barrier of window j - 1.
-    u32x4 bring[2][NG];                                       // window w travels in bring[w & 1]
-    auto stage_load = [&](u32x4 (&br)[NG], int w) {           // window index inside the slice
-        const size_t k0 = (size_t)(wbeg + w) * (KW * 32);
+    ScaleRow srows[PR];
 #pragma unroll
-        for (int i = 0; i < NG; ++i) br[i] = ld_global_u32x4(p.B + boff[i] + k0);
-    };
-    auto stage_store = [&](const u32x4 (&br)[NG], int base) {
-#pragma unroll
-        for (int i = 0; i < NG; ++i) win[base + st_idx + st_off(i)] = br[i];
-    };
-    WeightFrag<FP8> wf[2][KW][R];
-    float sc[2];                                              // a window lies inside one 128-wide scale block
-    auto issue_a = [&](int slot, int w, int t) {              // tile t of window w
-        const int tile = (wbeg + w) * KW + t;
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-            if constexpr (FP8) wf[slot][t][r].v = *reinterpret_cast<const u32x2 *>(abase[r] + (size_t)tile * 512 + lane_off);
-            else wf[slot][t][r].v = ld_global_u32x4(abase[r] + (size_t)tile * 1024 + lane_off);
-        }
-        if (FP8 && t == KW - 1) sc[slot] = scale_at(srow, tile >> 2);   // after the last use of the slot's previous scale
-    };
-    u32x4 b0[TB], b1[TB];
-    auto rd = [&](u32x4 (&b)[TB], int base, int t, int s) {
-#pragma unroll
-        for (int tb = 0; tb < TB; ++tb) {
-            b[tb] = win[base + t * TS + (tb * 4 + 2 * s) * 33 + ld_idx];
-        }
-    };
-    // a[2 pr + s]: row pair pr, k half s
-    auto mm = [&](const u32x4 (&a)[R], const u32x4 (&b)[TB], int s) {
-#pragma unroll
-        for (int tb = 0; tb < TB; ++tb)
-#pragma unroll
-            for (int pr = 0; pr < PR; ++pr) {
-                acc[pr][tb] = T::mfma32(a[2 * pr + s], b[tb], acc[pr][tb]);
-            }
-    };
-    auto operands = [&](u32x4 (&a)[R], int slot, int t) {
-        float s4[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) s4[r] = FP8 ? sc[slot] : 1.f;
-        weight_operands<FP8, R>(a, wf[slot][t], s4);
-        pair_to_rows32(a[0], a[1]);
-        if constexpr (PR == 2) pair_to_rows32(a[2], a[3]);
-    };
-    int cur = 0;                                              // LDS granule offset of the current window's buffer
-    // SLOT: weight slot; NEXT / NEXT2: windows j + 1 / j + 2 exist (compile-time, so the steady loop has no tests)
-    auto window = [&](auto slot_c, auto next_c, auto next2_c, int j) {
-        constexpr int slot = decltype(slot_c)::value;
-        constexpr bool NEXT = decltype(next_c)::value, NEXT2 = decltype(next2_c)::value;
-        const int nxt = cur == 2 * WG ? 0 : cur + WG;
-        u32x4 a[R];
-        auto half = [&](auto hs_c, const u32x4 (&use)[TB], u32x4 (&other)[TB]) {
-            constexpr int hs = decltype(hs_c)::value, t = hs >> 1, sh = hs & 1;
-            if (sh == 0) operands(a, slot, t);
-            if (hs < 2 * KW - 1) rd(other, cur, (hs + 1) >> 1, (hs + 1) & 1);
-            else if (NEXT) rd(other, nxt, 0, 0);
-            if (hs == 0 && NEXT2) stage_load(bring[slot], j + 2);
-            if (sh == 0 && t > 0 && NEXT2) issue_a(slot, j + 2, t - 1);   // the registers of tile t - 1 are free again
-            mm(a, use, sh);
-            // one scheduling region: the LDS reads and global loads above go out between the MFMAs
-#pragma unroll
-            for (int i = 0; i < TB; ++i) {
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);   // MFMA
-                __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);   // LDS read
-                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);   // global load
-            }
-            __builtin_amdgcn_sched_barrier(0);
-            if (hs == 2 * KW - 1 && NEXT2) issue_a(slot, j + 2, KW - 1);
-            if (hs == KW - 1) {
-                if (NEXT) stage_store(bring[slot ^ 1], nxt);
-                __syncthreads();
-            }
-        };
-        half(std::integral_constant<int, 0>{}, b0, b1);
-        half(std::integral_constant<int, 1>{}, b1, b0);
-        half(std::integral_constant<int, 2>{}, b0, b1);
-        half(std::integral_constant<int, 3>{}, b1, b0);
-        if constexpr (KW == 4) {
-            half(std::integral_constant<int, 4>{}, b0, b1);
-            half(std::integral_constant<int, 5>{}, b1, b0);
-            half(std::integral_constant<int, 6>{}, b0, b1);
-            half(std::integral_constant<int, 7>{}, b1, b0);
-        }
-        cur = nxt;
-    };
-    using I0 = std::integral_constant<int, 0>;
-    using I1 = std::integral_constant<int, 1>;
-    using Yes = std::true_type;
-    using No = std::false_type;
-
-    if (nwin > 0) {
-        stage_load(bring[0], 0);
-#pragma unroll
-        for (int t = 0; t < KW; ++t) issue_a(0, 0, t);
-        stage_store(bring[0], 0);
-        if (nwin > 1) {
-            stage_load(bring[1], 1);
-#pragma unroll
-            for (int t = 0; t < KW; ++t) issue_a(1, 1, t);
-        }
-        __syncthreads();
-        rd(b0, 0, 0, 0);
-        int j = 0;
-        for (; j + 3 < nwin; j += 2) {
-            window(I0{}, Yes{}, Yes{}, j);
-            window(I1{}, Yes{}, Yes{}, j + 1);
-        }
-        const int rem = nwin - j;                             // 1, 2 or 3
-        if (rem == 3) {
-            window(I0{}, Yes{}, Yes{}, j);
-            window(I1{}, Yes{}, No{}, j + 1);
-            window(I0{}, No{}, No{}, j + 2);
-        } else if (rem == 2) {
-            window(I0{}, Yes{}, No{}, j);
-            window(I1{}, No{}, No{}, j + 1);
-        } else {
-            window(I0{}, No{}, No{}, j);
-        }
-    }
-    mfma_settle();
+    for (int pr = 0; pr < PR; ++pr) srows[pr] = srow;          // the row groups of a wave lie in one 128-row block
+    PanelLoop<T, FP8, TB, PR>::run(acc, abase, srows, p.B, boff, wbeg, nwin, win);
 
     // accumulator element 4 g + e of lane 32 h + c: weight row 8 g + 4 h + e of the pair's 32, token c of the block's 32
     const int half = lane >> 5, c32 = lane & 31;

@@ -28,14 +28,28 @@ from .. import ops, arg_selector
 GEMV_TABLES = {"gemv_fp16": torch.float16, "gemv_bf16": torch.bfloat16, "gemv_soft_fp8": None}
 GEMM_TABLES = {"layoutA_gemm": ("rowmajor", torch.float16), "layoutA_soft_fp8_gemm": ("fp8", torch.bfloat16),
                "continuous_gemm": ("continuous", torch.bfloat16), "layout_gemm": ("native", torch.bfloat16)}
+# weight shapes (rows x K): the benchmark configurations, then the model lists the reference's scripts scan
+# (benchmark_and_test/gemv_benchmark.py:122-137): Llama2-7B, Qwen2-7B, DeepSeek-R1
+BENCH_16BIT = [(4096, 4096), (11008, 4096), (8192, 8192), (28672, 4096), (4096, 14336)]
+BENCH_FP8 = [(28672, 8192), (4096, 4096), (8192, 8192)]
+LLAMA2_7B = [(32000, 4096), (12288, 4096), (4096, 4096), (22016, 4096), (4096, 11008)]
+QWEN2_7B = [(37888, 3584), (4608, 3584), (3584, 3584), (3584, 18944)]
+DEEPSEEK_R1 = [(2112, 7168), (3072, 1536), (7168, 2048), (7168, 256), (512, 7168), (4608, 7168), (7168, 2304)]
+MODEL_SHAPES = LLAMA2_7B + QWEN2_7B + DEEPSEEK_R1
+
+
+def _unique(shapes):
+    return list(dict.fromkeys(shapes))
+
+
 DEFAULT_SHAPES = {
-    "gemv_fp16": [(11008, 4096), (4096, 4096), (4096, 11008)],
-    "gemv_bf16": [(4096, 4096), (28672, 8192), (8192, 8192), (28672, 4096), (4096, 14336)],
-    "gemv_soft_fp8": [(28672, 8192), (4096, 4096), (8192, 8192)],
-    "layoutA_gemm": [(11008, 4096), (4096, 4096), (4096, 11008)],
-    "layoutA_soft_fp8_gemm": [(28672, 8192), (4096, 4096)],
-    "continuous_gemm": [(8192, 8192), (11008, 4096)],
-    "layout_gemm": [(8192, 8192), (11008, 4096)],
+    "gemv_fp16": _unique([(11008, 4096), (4096, 4096), (4096, 11008)] + MODEL_SHAPES),
+    "gemv_bf16": _unique(BENCH_16BIT + [(28672, 8192)] + MODEL_SHAPES),
+    "gemv_soft_fp8": _unique(BENCH_FP8 + MODEL_SHAPES),
+    "layoutA_gemm": _unique([(11008, 4096), (4096, 4096), (4096, 11008)] + MODEL_SHAPES),
+    "layoutA_soft_fp8_gemm": _unique(BENCH_FP8[:2] + MODEL_SHAPES),
+    "continuous_gemm": _unique([(8192, 8192), (11008, 4096)] + MODEL_SHAPES),
+    "layout_gemm": _unique([(8192, 8192), (11008, 4096)] + MODEL_SHAPES),
 }
 DEFAULT_TOKENS = {"layoutA_gemm": [1, 8, 16, 32, 48, 64], "layoutA_soft_fp8_gemm": [1, 4, 16, 32, 64],
                   "continuous_gemm": [16, 32, 64], "layout_gemm": [16, 32, 64]}
@@ -92,7 +106,7 @@ def _gate(got, want):
     return bool((err <= 1e-2 + 1e-2 * want.abs()).all())
 
 
-def scan_gemv(table, shapes, iters):
+def scan_gemv(table, shapes, iters, progress=None):
     dtype = GEMV_TABLES[table]
     fp8 = dtype is None
     xdt = torch.bfloat16 if fp8 else dtype
@@ -106,30 +120,38 @@ def scan_gemv(table, shapes, iters):
         w0 = plain[0].view(torch.float8_e4m3fn).float() if fp8 else plain[0].float()
         want = x.float() @ w0.t()
         best = None
-        for block in (256, 512, 1024):
-            for p1 in (1, 2, 4):
-                if (block // 64) % p1 or (n // 16) % p1:
-                    continue
-                for p2 in (2, 4, 6, 8):
-                    def call(a):
-                        return lambda: ops.gemv_layoutA_wapper(a, x, n, k, 1, 0, block, 1, p1, p2, scale, None)
-                    if not _gate(call(packed[0])(), want):
-                        continue
-                    us = _time_graph([call(a) for a in packed], iters)
-                    if best is None or us < best[0]:
-                        best = (us, block, 1, p1, p2)
-        print("%s %dx%d -> %s" % (table, n, k, best), file=sys.stderr)
+        # kernel 1: (threads, row groups per workgroup, loads in flight); kernels 2 and 3 (soft-FP8 only):
+        # (threads, workgroups per CU, loads in flight)
+        grid = [(block, 1, p1, p2) for block in (256, 512, 1024) for p1 in (1, 2, 4) for p2 in (2, 4, 6, 8)
+                if (block // 64) % p1 == 0 and (n // 16) % p1 == 0]
+        grid += [(block, kid, per_cu, p2) for kid in ((2, 3) if fp8 else (2,)) for block in (256, 512, 1024)
+                 for per_cu in (1, 2, 4) for p2 in (2, 4) if block * per_cu <= 2048 and block * per_cu >= 512]
+        for block, kid, p1, p2 in grid:
+            def call(a):
+                return lambda: ops.gemv_layoutA_wapper(a, x, n, k, 1, 0, block, kid, p1, p2, scale, None)
+            if not _gate(call(packed[0])(), want):
+                continue
+            us = _time_graph([call(a) for a in packed], iters)
+            if best is None or us < best[0]:
+                best = (us, block, kid, p1, p2)
+        print("%s %dx%d -> %s" % (table, n, k, best), file=sys.stderr, flush=True)
         rows.append("%d,%d,%d,%d,%d,%d" % (n, k, best[1], best[2], best[3], best[4]))
+        if progress is not None:
+            progress(rows[-1])
         del plain, packed
     return rows
 
 
-def scan_gemm(table, shapes, tokens, iters):
+def scan_gemm(table, shapes, tokens, iters, progress=None):
     mode, dtype = GEMM_TABLES[table]
     fp8 = mode == "fp8"
     gen = torch.Generator(device="cuda").manual_seed(2025)
     rows = []
     for n, k in shapes:
+        if n % 128 or k % 128:
+            print("%s %dx%d skipped: the GEMM entry points need rows and K in multiples of 128" % (table, n, k),
+                  file=sys.stderr)
+            continue
         plain = _weights(n, k, dtype, fp8, _copies(n * k * (1 if fp8 else 2)), gen)
         packed = [ops.pack_layout_a(w) for w in plain]
         w0 = plain[0].view(torch.float8_e4m3fn).float() if fp8 else plain[0].float()
@@ -181,8 +203,10 @@ def scan_gemm(table, shapes, tokens, iters):
                     us = _time_graph([call(a) for a in packed], iters)
                     if best is None or us < best[0]:
                         best = (us, kid, p1, p2, p3)
-            print("%s %dx%d M=%d -> %s" % (table, n, k, m, best), file=sys.stderr)
+            print("%s %dx%d M=%d -> %s" % (table, n, k, m, best), file=sys.stderr, flush=True)
             rows.append("%d,%d,%d,%d,%d,%d,%d" % (n, m, k, best[1], best[2], best[3], best[4]))
+            if progress is not None:
+                progress(rows[-1])
         del plain, packed
     return rows
 
@@ -199,21 +223,26 @@ def main():
     for table in tables:
         shapes = DEFAULT_SHAPES[table] if args.shapes is None else \
             [tuple(int(v) for v in s.split("x")) for s in args.shapes.split(",")]
-        if table in GEMV_TABLES:
-            rows = scan_gemv(table, shapes, args.iters)
-            header = "m,k,BLOCK_DIM_X,KernelId,KernelParam1,KernelParam2"
-        else:
-            tokens = DEFAULT_TOKENS[table] if args.tokens is None else [int(v) for v in args.tokens.split(",")]
-            rows = scan_gemm(table, shapes, tokens, args.iters)
-            header = "m,n,k,kernelId,kernelParam1,kernelParam2,kernelParam3"
+        gemv = table in GEMV_TABLES
+        header = "m,k,BLOCK_DIM_X,KernelId,KernelParam1,KernelParam2" if gemv else \
+            "m,n,k,kernelId,kernelParam1,kernelParam2,kernelParam3"
         if args.update:
             path = arg_selector.selector(table).path()
-            with open(path, "a") as f:
-                f.write("\n".join(rows) + "\n")
+            out = open(path, "a")
         else:
             path = "%s_scan_best_args.csv" % table
-            with open(path, "w") as f:
-                f.write(header + "\n" + "\n".join(rows) + "\n")
+            out = open(path, "w")
+            out.write(header + "\n")
+
+        def progress(row):               # rows reach the file as they are found
+            out.write(row + "\n")
+            out.flush()
+        if gemv:
+            rows = scan_gemv(table, shapes, args.iters, progress)
+        else:
+            tokens = DEFAULT_TOKENS[table] if args.tokens is None else [int(v) for v in args.tokens.split(",")]
+            rows = scan_gemm(table, shapes, tokens, args.iters, progress)
+        out.close()
         print("wrote %d rows to %s" % (len(rows), path), file=sys.stderr)
 
 

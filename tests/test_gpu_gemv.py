@@ -111,3 +111,63 @@ def test_gemv_errors(mlk):
         mlk.gemv_layoutA(a.view(2, 4, 128), torch.zeros(1, 32, dtype=torch.bfloat16, device="cuda"))
     with pytest.raises(RuntimeError, match="data type"):
         mlk.gemv_layoutA(a, torch.zeros(1, 32, dtype=torch.float16, device="cuda"))
+
+
+@pytest.mark.parametrize("kind", ["bf16", "fp16", "fp8", "fp8_matrix_cores"])
+@pytest.mark.parametrize("n,k,block,per_cu,depth", [
+    (4096, 4096, 1024, 1, 2),      # one row group per workgroup
+    (11008, 4096, 512, 2, 4),      # uneven deal: two or three row groups per workgroup
+    (28672, 2048, 256, 1, 8),      # seven row groups per workgroup, several 128-row scale blocks each
+    (48, 192, 1024, 4, 2),         # fewer row groups than workgroups asked for, fewer tiles than waves
+    (2112, 7168, 512, 4, 6),       # tiles not a multiple of the wave count
+])
+def test_gemv_persistent_kernels(mlk, kind, n, k, block, per_cu, depth):
+    """Kernel id 2 (one uninterrupted stream per wave over a range of row groups) and, for soft-FP8 weights,
+    kernel id 3 (the same with the products on the matrix cores) against the oracle, for 1 to 4 tokens."""
+    fp8 = kind.startswith("fp8")
+    if fp8 and k % 64:
+        pytest.skip("soft-FP8 tiles cover 64 k")
+    dtype = torch.float16 if kind == "fp16" else torch.bfloat16
+    kid = 3 if kind == "fp8_matrix_cores" else 2
+    scale = None
+    if fp8:
+        codes = fp8_codes((n, k), 77)
+        g = torch.Generator().manual_seed(78)
+        scale = (torch.rand(((n + 127) // 128, (k + 127) // 128), generator=g) * 0.02 + 0.001).float()
+        a = pack_a(codes).cuda()
+    else:
+        w = randn((n, k), dtype, 0.02, 77)
+        a = pack_a(w).cuda()
+    for m in (1, 3, 4):
+        x = randn((m, k), dtype, 1.0, 80 + m)
+        bias = randn((1, n), dtype, 1.0, 90 + m)
+        y = mlk.gemv_layoutA_wapper(a, x.cuda(), n, k, alpha=0.75, blockDimX=block, kernelId=kid, kernelParam1=per_cu,
+                                    kernelParam2=depth, scale_matrix=None if scale is None else scale.cuda(),
+                                    bias=bias.cuda())
+        if fp8:
+            want = ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), x, 0.75, bias)
+        else:
+            want = ogemm.linear_expected(w, x, 0.75, bias)
+        assert_close(y, want, RTOL, ATOL, "persistent gemv %s M=%d" % (kind, m))
+        y2 = mlk.gemv_layoutA_wapper(a, x.cuda(), n, k, alpha=0.75, blockDimX=block, kernelId=kid, kernelParam1=per_cu,
+                                     kernelParam2=depth, scale_matrix=None if scale is None else scale.cuda(),
+                                     bias=bias.cuda())
+        assert torch.equal(y, y2)
+
+
+def test_gemv_matrix_core_variant_all_codes_exact(mlk):
+    """Kernel id 3 widens with the same instructions as the other kernels: every finite e4m3 code comes back
+    exactly through a one-hot activation vector (one code per weight row, in even and odd rows and octets)."""
+    k = 128
+    codes = torch.tensor([c for c in range(256) if c not in (0x7F, 0xFF)] + [0, 0], dtype=torch.uint8)
+    for col in (5, 8, 77, 127):
+        w = torch.zeros((256, k), dtype=torch.uint8)
+        w[:, col] = codes
+        x = torch.zeros((1, k), dtype=torch.bfloat16)
+        x[0, col] = 1.0
+        for s in (1.0, 0.37, 0.5):
+            scale = torch.full((2, 1), s, dtype=torch.float32)
+            y = mlk.gemv_layoutA_wapper(pack_a(w).cuda(), x.cuda(), 256, k, blockDimX=256, kernelId=3, kernelParam1=1,
+                                        kernelParam2=2, scale_matrix=scale.cuda())
+            want = softfp8.bf16_bits_to_f32(softfp8.dequant_bf16_bits(codes.numpy(), np.float32(s)))
+            assert np.array_equal(y.cpu().float().numpy().reshape(-1), want)

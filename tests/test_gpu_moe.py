@@ -201,6 +201,30 @@ def test_fused_moe_soft_fp8(mlk, T):
     _moe_case(mlk, T, 8, 2, 256, 384, torch.bfloat16, 300 + T, fp8=True)
 
 
+@pytest.mark.parametrize("T,E,K,H,I", [
+    (256, 8, 2, 256, 384),      # six token blocks per task: panels of 96 tokens
+    (300, 4, 2, 512, 384),      # eight blocks (panels of 128 tokens), then a pass of 44 tokens on the row-shared kernels
+    (200, 2, 1, 768, 128),      # one k window per slice boundary case: I = 128
+    (256, 3, 3, 256, 1024),     # every token on every expert: tasks of 256 tokens in two panels each
+])
+def test_fused_moe_soft_fp8_panel_kernels(mlk, T, E, K, H, I):
+    """Soft-FP8 weights with more than 64 tokens per pass over an expert run the panel kernels (32x32x16 products);
+    switching them off (experiment switch 9) must give the row-shared kernels' result to the same tolerance."""
+    from muxi_native_layout_kernels_amd import _lib
+    import ctypes
+    lib = _lib.load()
+    plan = (ctypes.c_int32 * 8)()
+    assert lib.mlk_moe_plan(T, E, K, H, I, 2, ctypes.addressof(plan)) == 0 and plan[0] == 4, "this case must take the panel path"
+    y1 = _moe_case(mlk, T, E, K, H, I, torch.bfloat16, 2100 + T, fp8=True)
+    lib.mlk_set_tunable(9, 1)
+    try:
+        assert lib.mlk_moe_plan(T, E, K, H, I, 2, ctypes.addressof(plan)) == 0 and plan[0] == 3
+        y2 = _moe_case(mlk, T, E, K, H, I, torch.bfloat16, 2100 + T, fp8=True)
+    finally:
+        lib.mlk_set_tunable(9, 0)
+    assert_close(y1, y2.double().cpu().numpy(), RTOL, ATOL, "panel kernels vs row-shared kernels")
+
+
 def test_fused_moe_grouped_sigmoid_bias(mlk):
     E = 64
     bias = randn((E,), torch.bfloat16, 0.05, 9).abs()

@@ -146,7 +146,7 @@ def test_moe_plan_fits_the_workgroup_lds_for_every_token_count(E, K, H, I, kind)
     than one row group per wave was chosen."""
     for T in range(1, 257):
         p = _plan(T, E, K, H, I, kind)
-        assert p["path"] in (0, 1, 2, 3) and p["cb"] in (1, 2, 3, 4, 6, 8)
+        assert p["path"] in (0, 1, 2, 3, 4) and p["cb"] in (1, 2, 3, 4, 6, 8)
         if p["path"] in (1, 2):
             assert p["down_lds"] + p["static_lds"] <= 64 * 1024, (T, p)
             assert p["down_wk"] >= 1 and p["down_lds"] == p["down_wk"] * p["down_r"] * p["cb"] * 1024 + T * 16 * p["down_r"] * 4
@@ -155,6 +155,9 @@ def test_moe_plan_fits_the_workgroup_lds_for_every_token_count(E, K, H, I, kind)
                 assert (H // 16) % p["down_r"] == 0 and (I // 32) % p["down_r"] == 0
         if p["path"] == 3:
             assert p["cb"] >= 2 and (I // 32) % (p["down_slices"] * (2 if p["cb"] > 4 else 4)) == 0
+        if p["path"] == 4:          # panel kernels: output rows in tiles of 256, at least four k windows per slice
+            assert kind == 2 and p["cb"] >= 5 and H % 256 == 0 and 1 <= p["down_slices"] <= 8
+            assert p["down_slices"] == 1 or (I // 128) // p["down_slices"] >= 4
         assert p["path"] != 0 or T == 1
 
 
@@ -171,5 +174,9 @@ def test_moe_plan_known_cases():
     assert _plan(16, 8, 2, 4096, 14336, 1)["path"] == 1
     assert _plan(64, 8, 2, 4096, 14336, 1)["path"] == 3
     assert _plan(256, 8, 2, 4096, 14336, 1)["path"] == 3
+    # soft-FP8 with more than 64 tokens per pass over an expert: panel kernels, if the output rows tile in 256
+    assert _plan(64, 8, 2, 4096, 14336, 2)["path"] == 3
+    assert _plan(256, 8, 2, 4096, 14336, 2)["path"] == 4
+    assert _plan(256, 8, 2, 4096 + 128, 14336, 2)["path"] == 3
     # 500 tokens run as 256 + 244: the plan of the first pass is what the query reports
     assert _plan(500, 256, 8, 7168, 256, 2) == _plan(256, 256, 8, 7168, 256, 2)
