@@ -136,9 +136,12 @@ def main():
         row = dict(name=name, us=t["us"], us_median=t["us_median"], us_min=t["us_min"], bytes=algo,
                    gbps=algo / t["us"] / 1e3, frac=algo / t["us"] / 1e3 / HBM_PEAK_GBPS, wall=t["wall"])
         row.update(extra)
-        if name in traffic_table:
-            row["traffic"] = traffic_table[name]
-            row["traffic_over_algorithmic"] = traffic_table[name] / algo
+        got = traffic_table.get(name)
+        if isinstance(got, dict):   # counted for one routing: valid only when this run drew as many active experts
+            got = got["bytes"] if got.get("active_experts") == extra.get("active_experts") else None
+        if got is not None:
+            row["traffic"] = got
+            row["traffic_over_algorithmic"] = got / algo
         return row
 
     def read_only_us(nbytes, steps, shapes=((512, 1024), (1024, 512), (256, 2048), (512, 512), (1024, 256))):
