@@ -131,7 +131,14 @@ struct TileLoop {
                 }
         };
         auto step = [&](int slot, bool do_stage, bool do_issue) {
+            // The activation loads of the next window go out before the products of this one: left alone the
+            // compiler sinks them to their first use, the parking stores below.  (Loads return in order, so the
+            // wait before those stores is also the wait for the weights requested at the end of the previous
+            // step.  Deeper weight rings, with the lead-in arranged so that the loop is entered in its own
+            // steady state and no trip drains the queue, measured slower: a CU keeps a bounded number of requests
+            // in flight, and queueing more of them does not raise it.)
             if (do_stage) stage_load();
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int w = 0; w < KW; ++w) {
                 // all fragment reads of the k tile go out first, then the products (the tests on nb
