@@ -294,32 +294,55 @@ __global__ void __launch_bounds__(1024) moe_align_kernel(const int32_t *__restri
     }
     __syncthreads();
 
-    // totals -> padded prefix (one thread; E <= 256) ; per-wave cursors
-    if (tid == 0) {
-        int run = 0, nt = 0;
-        for (int e = 0; e < E; ++e) {
-            int total = 0;
-            for (int w = 0; w < NW; ++w) total += cnt[w][e];
-            start[e] = run;
-            int nb = (total + 15) >> 4;
-            for (int b = 0; b < nb; ++b) experts_ids[(run >> 4) + b] = e;
-            if (tasks) {
-                for (int b = 0; b < nb; b += cb_max) {
-                    MoeTask tk;
-                    tk.expert = e;
-                    tk.block0 = (run >> 4) + b;
-                    tk.nblocks = min(cb_max, nb - b);
-                    tk.pad = 0;
-                    tasks[nt++] = tk;
-                }
-            }
-            run += nb << 4;
-            cumsum_out[e] = start[e] + total;          // where the reference's atomic cursor ends up
+    // totals -> padded prefix and task list, one thread per expert (E <= 256): inclusive scans of the padded
+    // sizes and of the task counts through LDS, then every expert writes its own blocks and tasks
+    __shared__ int scan_pad[kMaxExperts], scan_task[kMaxExperts];
+    int total = 0, nb = 0, ntk = 0;
+    if (tid < E) {
+        for (int w = 0; w < NW; ++w) total += cnt[w][tid];
+        nb = (total + 15) >> 4;
+        ntk = (nb + cb_max - 1) / cb_max;
+        scan_pad[tid] = nb << 4;
+        scan_task[tid] = ntk;
+    }
+    __syncthreads();
+    for (int d = 1; d < E; d <<= 1) {
+        int a = 0, c = 0;
+        if (tid < E && tid >= d) {
+            a = scan_pad[tid - d];
+            c = scan_task[tid - d];
         }
-        start[E] = run;
-        cumsum_out[E] = run;
-        padded_blocks[0] = run >> 4;
-        if (n_tasks) n_tasks[0] = nt;
+        __syncthreads();
+        if (tid < E && tid >= d) {
+            scan_pad[tid] += a;
+            scan_task[tid] += c;
+        }
+        __syncthreads();
+    }
+    if (tid < E) {
+        const int e = tid;
+        const int run = scan_pad[e] - (nb << 4);        // exclusive
+        start[e] = run;
+        for (int b = 0; b < nb; ++b) experts_ids[(run >> 4) + b] = e;
+        if (tasks) {
+            int nt = scan_task[e] - ntk;
+            for (int b = 0; b < nb; b += cb_max) {
+                MoeTask tk;
+                tk.expert = e;
+                tk.block0 = (run >> 4) + b;
+                tk.nblocks = min(cb_max, nb - b);
+                tk.pad = 0;
+                tasks[nt++] = tk;
+            }
+        }
+        cumsum_out[e] = run + total;                    // where the reference's atomic cursor ends up
+        if (e == E - 1) {
+            const int end = scan_pad[e];
+            start[E] = end;
+            cumsum_out[E] = end;
+            padded_blocks[0] = end >> 4;
+            if (n_tasks) n_tasks[0] = scan_task[e];
+        }
     }
     __syncthreads();
     for (int e = tid; e < E; e += 1024) {
