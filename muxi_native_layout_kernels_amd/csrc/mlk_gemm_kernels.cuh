@@ -169,7 +169,9 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
             if (FP8) sc[slot] = scale_at(srow, kt >> 2);
         };
         auto step = [&](int slot, int buf, bool do_stage, bool do_issue) {
+            // pinned ahead of the products: the compiler would sink these loads to the parking stores below
             if (do_stage) stage_load();
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = win[buf * win_granules + (wave * CB + cb) * 68 + q * 17 + r16];
             consume(slot);
@@ -178,18 +180,33 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
             if (do_stage) stage_store(buf ^ 1);
             __syncthreads();
         };
+        // (Loads return in order, so the wait before the parking stores is also the wait for the weights requested
+        // at the end of the previous step: two slots behave like one window in flight across the barrier.  Three
+        // slots with the activations requested ahead of the youngest weights, so that two windows stay in flight,
+        // measured 10 % slower at 40 to 64 tokens: more requests in flight per CU do not raise its bandwidth.)
         static_assert(U % 2 == 0, "the staged loop alternates two LDS buffers inside a U-step unroll");
         if (nwin > 0) {
             stage_load();
             stage_store(0);
-#pragma unroll
-            for (int u = 0; u < U; ++u)
-                if (u < nwin) issue_a(u);
-            __syncthreads();
             int j = 0;
-            for (; j + 2 * U <= nwin; j += U) {
+            if (nwin >= 2 * U) {
+                // Lead-in of the unrolled loop: all U windows requested without conditions and the first one
+                // waited for, which is the state every trip of the loop leaves behind (U - 1 windows in flight,
+                // the current one landed).  Entered in any other state the loop would be compiled to wait for
+                // all of its loads at the top of every trip.
 #pragma unroll
-                for (int u = 0; u < U; ++u) step(u, u & 1, true, true);
+                for (int u = 0; u < U; ++u) issue_a(u);
+                asm volatile("" ::"v"(wf[0][R - 1].v));
+                __syncthreads();
+                for (; j + 2 * U <= nwin; j += U) {
+#pragma unroll
+                    for (int u = 0; u < U; ++u) step(u, u & 1, true, true);
+                }
+            } else {
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (u < nwin) issue_a(u);
+                __syncthreads();
             }
 #pragma unroll
             for (int u = 0; u < U; ++u)
@@ -328,9 +345,11 @@ __global__ void __launch_bounds__(wave_kernel_threads(R *CB, U, STAGE)) gemm_wav
 
 // Kernel id 4: one workgroup per CU, the row groups dealt out as evenly as possible, so a workgroup
 // owns floor or ceil(groups / grid) consecutive row groups: RMAX or RMAX - 1.  Both cases run the
-// fully unrolled body; the test is uniform for the workgroup.  Row-major operands, no K split.
-template <class T, int CB, int RMAX, int U>
-__global__ void __launch_bounds__(wave_kernel_threads(RMAX *CB, U, false)) gemm_wave_balanced_kernel(GemmArgs p) {
+// fully unrolled body; the test is uniform for the workgroup.  Row-major operands, no K split.  STAGE: the
+// activations of a window of WK k tiles are fetched once per workgroup and shared by all its row groups through
+// LDS (three and four token blocks).
+template <class T, int CB, int RMAX, int U, bool STAGE = false>
+__global__ void __launch_bounds__(wave_kernel_threads(RMAX *CB, U, STAGE)) gemm_wave_balanced_kernel(GemmArgs p) {
     extern __shared__ f32x4 red[];
     __shared__ int s_last;
     const int groups = p.N >> 4;
@@ -338,9 +357,9 @@ __global__ void __launch_bounds__(wave_kernel_threads(RMAX *CB, U, false)) gemm_
     const int rg0 = (int)((long long)rt * groups / (int)gridDim.x);
     const int nr = (int)((long long)(rt + 1) * groups / (int)gridDim.x) - rg0;
     if (nr == RMAX)
-        gemm_wave_body<T, false, CB, RMAX, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR, U, false>(p, rt, 0, rg0, gridDim.x, red, s_last);
+        gemm_wave_body<T, false, CB, RMAX, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR, U, STAGE>(p, rt, 0, rg0, gridDim.x, red, s_last);
     else
-        gemm_wave_body<T, false, CB, RMAX - 1, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR, U, false>(p, rt, 0, rg0, gridDim.x, red, s_last);
+        gemm_wave_body<T, false, CB, RMAX - 1, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR, U, STAGE>(p, rt, 0, rg0, gridDim.x, red, s_last);
 }
 
 // Kernel 2: row-shared tile kernel (see mlk_tile.cuh).  Four waves per workgroup, R row groups
@@ -511,6 +530,19 @@ static int launch_balanced(const GemmArgs &p, int wgs, hipStream_t s) {
     constexpr int U = RMAX * CB <= 4 ? 4 : (RMAX * CB <= 8 ? 3 : 2);     // k tiles in flight per wave
     GemmArgs q = p;
     q.SK = 1;
+    if constexpr (CB >= 3) {
+        // three and four token blocks: the activations of a window of WK k tiles are staged once per workgroup
+        // in LDS and shared by all its row groups (WK waves, one k tile of the window each)
+        while (q.WK > 4) q.WK >>= 1;
+        const int tiles_total = q.K / 32;
+        const size_t win_bytes = (size_t)2 * q.WK * CB * 68 * 16;
+        size_t lds = (size_t)q.WK * RMAX * CB * 1024;
+        if (win_bytes > lds) lds = win_bytes;
+        if (q.WK < 2 || tiles_total % q.WK != 0 || lds > 64 * 1024) return 1;      // does not apply: the caller falls back
+        gemm_wave_balanced_kernel<T, CB, RMAX, 2, true><<<wgs, q.WK * 64, lds, s>>>(q);
+        MLK_LAUNCH_CHECK();
+        return MLK_OK;
+    }
     while (q.WK * 64 > wave_kernel_threads(RMAX * CB, U, false) || (size_t)q.WK * RMAX * CB * 1024 > 64 * 1024) q.WK >>= 1;
     size_t lds = q.WK > 1 ? (size_t)q.WK * RMAX * CB * 1024 : 0;
     gemm_wave_balanced_kernel<T, CB, RMAX, U><<<wgs, q.WK * 64, lds, s>>>(q);
@@ -524,7 +556,7 @@ static int balanced_grid(const GemmArgs &p, int CB, int *r_max) {
     const int groups = p.N / 16;
     if (groups <= cus) return 0;
     const int r = (groups + cus - 1) / cus;
-    if (r < 2 || r > 4 || CB > 2) return 0;   // from three token blocks on the row-shared kernel is faster
+    if (r < 2 || r > 4 || CB > 4) return 0;
     *r_max = r;
     return cus;
 }
@@ -539,10 +571,15 @@ static int launch_rc(const GemmArgs &p, int kernel_id, int R, int CB, hipStream_
         if (kernel_id == 4) {
             int r_max = 0;
             const int wgs = p.SK == 1 ? balanced_grid(p, CB, &r_max) : 0;
-#define MLK_BAL(CC, RR) \
-    if (wgs && CB == CC && r_max == RR) return launch_balanced<T, CC, RR>(p, wgs, s);
+#define MLK_BAL(CC, RR)                                              \
+    if (wgs && CB == CC && r_max == RR) {                            \
+        const int rc = launch_balanced<T, CC, RR>(p, wgs, s);        \
+        if (rc <= 0) return rc;                                      \
+    }
             MLK_BAL(1, 2) MLK_BAL(1, 3) MLK_BAL(1, 4)
             MLK_BAL(2, 2) MLK_BAL(2, 3) MLK_BAL(2, 4)
+            MLK_BAL(3, 2) MLK_BAL(3, 3) MLK_BAL(3, 4)
+            MLK_BAL(4, 2) MLK_BAL(4, 3) MLK_BAL(4, 4)
 #undef MLK_BAL
         }
     }

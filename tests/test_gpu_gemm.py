@@ -205,10 +205,11 @@ def test_gemm_panel_kernel_is_the_wide_default(mlk):
 
 
 @pytest.mark.parametrize("n", [16 * 300, 16 * 384, 16 * 688, 16 * 768, 16 * 1000])
-@pytest.mark.parametrize("m", [1, 7, 16, 32, 40])
+@pytest.mark.parametrize("m", [1, 7, 16, 32, 40, 48, 57, 64])
 def test_gemm_balanced_rows_kernel(mlk, n, m):
     """kernelId 4: one workgroup per CU, the row groups dealt out evenly (one to four per workgroup, uneven
-    deals included).  More than 32 tokens, or shapes it does not take, run as kernel 1."""
+    deals included).  From three token blocks on the activations of a k window are shared through LDS; shapes
+    it does not take run as kernel 1."""
     k = 256
     w = randn((n, k), torch.bfloat16, 0.05, 71)
     b = randn((m, k), torch.bfloat16, 1.0, 72)
@@ -218,6 +219,28 @@ def test_gemm_balanced_rows_kernel(mlk, n, m):
         c = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=2.0, kernelParam1=1, kernelParam2=p2, kernelParam3=1,
                                     kernelId=4, bias=bias.cuda())
         assert_close(c, ogemm.linear_expected(w, b, 2.0, bias), RTOL, ATOL, "balanced rows n=%d m=%d" % (n, m))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("k", [192, 1024, 1152, 4096])
+@pytest.mark.parametrize("m", [33, 48, 50, 64])
+def test_gemm_balanced_rows_kernel_shared_windows(mlk, dtype, k, m):
+    """kernelId 4 at three and four token blocks over short and long K: K = 192 (six k tiles, no whole
+    windows: the plain wave kernel takes it), 1024 and 4096 (the unrolled loop with its lead-in), 1152 (36 k
+    tiles: nine windows, an odd tail), on 688 row groups (three and two per workgroup on 256 CUs); twice, and the
+    two runs must agree bit for bit."""
+    n = 16 * 688
+    w = randn((n, k), dtype, 0.02, 74)
+    b = randn((m, k), dtype, 1.0, 75)
+    bias = randn((1, n), dtype, 1.0, 76)
+    a = pack_a(w).cuda()
+    for p2 in (4, 2):
+        c = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=1, kernelParam2=p2, kernelParam3=1,
+                                    kernelId=4, bias=bias.cuda())
+        assert_close(c, ogemm.linear_expected(w, b, 0.5, bias), RTOL, ATOL, "balanced shared k=%d m=%d p2=%d" % (k, m, p2))
+        c2 = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=1, kernelParam2=p2, kernelParam3=1,
+                                     kernelId=4, bias=bias.cuda())
+        assert torch.equal(c, c2)
 
 
 def test_gemm_balanced_rows_fallbacks(mlk):
