@@ -432,7 +432,7 @@ def main():
     if args.calibrate_copy:
         src = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
-        for _ in range(4):   # fp8_repack_kernel: one dword in, one dword out per thread
+        for _ in range(4):   # the repack kernel as a plain copy of known size: 16 bytes in and 16 bytes out per thread
             _lib.check(lib.mlk_fp8_weight_repack(src.data_ptr(), dst.data_ptr(), src.numel(),
                                                  torch.cuda.current_stream().cuda_stream), "copy")
         torch.cuda.synchronize()

@@ -61,6 +61,19 @@ def test_fp8_weight_repack(mlk, shape):
     assert torch.equal(mlk.fp8_weight_repack(out).cpu(), w)  # involution
 
 
+def test_fp8_weight_repack_tails_and_unaligned_views(mlk):
+    """Sizes that are not multiples of 16 bytes (the last one to three dwords take the dword kernel) and views
+    whose first byte is 4 or 8 bytes into an allocation (no 16-byte alignment: the dword kernel takes it all)."""
+    rng = np.random.default_rng(12)
+    for nbytes in (4, 12, 20, 4 * 1027, 16 * 513 + 8):
+        for lead in (0, 4, 8):
+            whole = torch.from_numpy(rng.integers(0, 255, size=lead + nbytes, dtype=np.uint8, endpoint=True)).cuda()
+            w = whole[lead:]
+            assert w.data_ptr() % 16 == lead
+            out = mlk.fp8_weight_repack(w)
+            assert np.array_equal(out.cpu().numpy(), layouts.fp8_weight_repack(w.cpu().numpy())), (nbytes, lead)
+
+
 def test_relayout_errors(mlk):
     with pytest.raises(RuntimeError, match="multiple of 16"):
         mlk.layoutB(torch.zeros(8, 32, dtype=torch.bfloat16, device="cuda"))
