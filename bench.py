@@ -255,7 +255,18 @@ def main():
         extra["cpu_baseline"] = cpu_linear(n, k, 1, kind, cpu_rows)
         return finish(name, t, algo, **extra)
 
-    def gemm_case(name, n, k, kind, m, steps, warmup, native=False, copies=None, cpu_rows=2048, cpu=True):
+    def blas_yardstick(row, n, k, dt, m, steps, count):
+        """torch.matmul (vendor BLAS) on `count` rotating un-packed copies of a weight matrix of the same shape."""
+        W = [(torch.randn((n, k), generator=gen, device=dev) * 0.02).to(dt) for _ in range(count)]
+        b = torch.randn((m, k), generator=gen, device=dev).to(dt)
+        out = torch.empty((m, n), dtype=dt, device=dev)
+        t = run_graph([(lambda w=w: torch.matmul(b, w.t(), out=out)) for w in W], steps, 3, reps=3)
+        row["blas_us"] = t["us_median"]
+        row["blas_note"] = ("torch.matmul (vendor BLAS) on %d rotating un-packed %s weight matrices of the same shape"
+                            % (count, str(dt).replace("torch.", "")))
+        del W
+
+    def gemm_case(name, n, k, kind, m, steps, warmup, native=False, copies=None, cpu_rows=2048, cpu=True, blas=False):
         xk = 1 if kind == 2 else kind
         A = weights(n, k, kind, copies or copies_for(n * k * (1 if kind == 2 else 2)))
         b = torch.randn((m, k), generator=gen, device=dev).to(DT[xk])
@@ -292,6 +303,10 @@ def main():
         row = finish(name, t, algo, params=[kid, p1, p2, p3], copies=len(A))
         if cpu:
             row["cpu_baseline"] = cpu_linear(n, k, m, kind, cpu_rows, native=native)
+        if blas and kind != 2:
+            count = len(A)
+            del A
+            blas_yardstick(row, n, k, DT[kind], m, min(steps, 100), count)
         return row
 
     def panel_case(name, n, k, kind, m, steps):
@@ -455,7 +470,7 @@ def main():
     # ------------------------------------------------------------ headline
     N, K_, M = 11008, 4096, 16
     HEAD = "C2 fp16 gemm_layoutA 11008x4096 M=16"
-    head = gemm_case(HEAD, N, K_, 0, M, args.steps, args.warmup)
+    head = gemm_case(HEAD, N, K_, 0, M, args.steps, args.warmup, blas=not args.quick)
     per_config = []
 
     def add(case, name, *a, **kw):
@@ -477,13 +492,13 @@ def main():
         short = max(20, min(args.steps, 100))
         add(gemv_case, "C1 bf16 gemv 4096x4096", 4096, 4096, 1, short, 10, yardstick=True, cpu_rows=4096)
         for m in (1, 8, 32, 64):
-            add(gemm_case, "C2 fp16 gemm_layoutA 11008x4096 M=%d" % m, N, K_, 0, m, short, 10)
+            add(gemm_case, "C2 fp16 gemm_layoutA 11008x4096 M=%d" % m, N, K_, 0, m, short, 10, blas=True)
         add(gemv_case, "C2 fp16 gemv 11008x4096", N, K_, 0, short, 10)
         add(gemv_case, "C3 soft-fp8 gemv 28672x8192", 28672, 8192, 2, short, 10, yardstick=True, cpu_rows=1024)
         for m in (4, 16):
             add(gemm_case, "C3 soft-fp8 gemm_layoutA 28672x8192 M=%d" % m, 28672, 8192, 2, m, short, 10, cpu_rows=1024)
         add(gemm_case, "C4 bf16 gemm_layoutABC+reLayoutC 8192x8192 M=32", 8192, 8192, 1, 32, short, 10, native=True,
-            cpu_rows=1024)
+            cpu_rows=1024, blas=True)
         add(relayout_case, "C4 layoutB bf16 [32, 8192]", "layoutB", short)
         add(relayout_case, "C4 reLayoutC bf16 [32, 8192]", "reLayoutC", short)
         add(relayout_case, "C3 fp8_weight_repack 28672x8192", "fp8_weight_repack", 10)
@@ -536,6 +551,8 @@ def main():
             "what": "pure streaming read (mlk_stream_read, 256 MiB x 4 rotating buffers) measured in this run",
             "us_for_one_launch_reading_the_headline_weights": round(same_size, 3)},
         "infinity_cache_resident": resident,
+        "vendor_blas": None if head.get("blas_us") is None else {
+            "us_per_call": round(head["blas_us"], 3), "what": head["blas_note"] + ", same token count, same graph-replay timing"},
         "cpu_baseline": head.get("cpu_baseline"),
         "per_config": per_config,
     }
