@@ -32,8 +32,9 @@ What the columns select on gfx950 (the rows are produced by the scripts in
                                  other values: chosen from the shape)
                              4 = kernel 1 with one workgroup per CU and the row groups dealt out
                                  evenly, two to four per workgroup (16-bit weights, row-major
-                                 operands, up to 64 tokens, N/16 above the CU count; from 33 tokens on
-                                 the activations of a k window are shared through LDS; kernelParam1
+                                 operands, up to 64 tokens, N/16 above the CU count; from 33 tokens on,
+                                 and from 17 tokens on with kernelParam2 = 8, the activations of a k
+                                 window are shared through LDS by up to eight waves; kernelParam1
                                  and kernelParam3 are not used; otherwise the same as 1)
                              12, 14, 16, 18 = kernel 1 with 2, 4, 6, 8 k tiles in flight per
                                  wave (up to 16 tokens, row-major activations and output;

@@ -349,7 +349,7 @@ __global__ void __launch_bounds__(wave_kernel_threads(R *CB, U, STAGE)) gemm_wav
 // activations of a window of WK k tiles are fetched once per workgroup and shared by all its row groups through
 // LDS (three and four token blocks).
 template <class T, int CB, int RMAX, int U, bool STAGE = false>
-__global__ void __launch_bounds__(wave_kernel_threads(RMAX *CB, U, STAGE)) gemm_wave_balanced_kernel(GemmArgs p) {
+__global__ void __launch_bounds__(STAGE ? 512 : wave_kernel_threads(RMAX *CB, U, STAGE)) gemm_wave_balanced_kernel(GemmArgs p) {
     extern __shared__ f32x4 red[];
     __shared__ int s_last;
     const int groups = p.N >> 4;
@@ -490,13 +490,14 @@ static int launch(const GemmArgs &p, hipStream_t s) {
     int row_tiles = (q.N / 16) / R;
     int grid = row_tiles * q.SK;
     size_t lds = q.WK > 1 ? (size_t)q.WK * R * CB * 1024 : 0;
-    if constexpr (BMODE == MLK_B_ROWMAJOR && CB >= 3) {
+    if constexpr (BMODE == MLK_B_ROWMAJOR && CB >= 2) {
         // stage row-major activations through LDS when every K slice is a whole number of WK-tile windows
         const int tiles_total = q.K / 32;
         const int tiles_per = (tiles_total + q.SK - 1) / q.SK;
         const size_t win_bytes = (size_t)2 * q.WK * CB * 68 * 16;
-        // (measured: staging pays only from three token blocks up; below that the direct gather wins)
-        if (g_tunable[1] && CB >= 3 && q.WK >= 2 && tiles_total % q.SK == 0 && tiles_per % q.WK == 0 && win_bytes <= 48 * 1024) {
+        // (measured: staging pays from three token blocks up, and at two token blocks with eight waves to share a
+        // window; below that the direct gather wins)
+        if (g_tunable[1] && (CB >= 3 || q.WK >= 8) && q.WK >= 2 && tiles_total % q.SK == 0 && tiles_per % q.WK == 0 && win_bytes <= 48 * 1024) {
             constexpr int US = (R * CB >= 8) ? 2 : 4;
             if (win_bytes > lds) lds = win_bytes;
             gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, US, true><<<grid, q.WK * 64, lds, s>>>(q);
@@ -530,18 +531,36 @@ static int launch_balanced(const GemmArgs &p, int wgs, hipStream_t s) {
     constexpr int U = RMAX * CB <= 4 ? 4 : (RMAX * CB <= 8 ? 3 : 2);     // k tiles in flight per wave
     GemmArgs q = p;
     q.SK = 1;
-    if constexpr (CB >= 3) {
-        // three and four token blocks: the activations of a window of WK k tiles are staged once per workgroup
-        // in LDS and shared by all its row groups (WK waves, one k tile of the window each)
-        while (q.WK > 4) q.WK >>= 1;
+    if (CB >= 3 || (CB == 2 && q.WK >= 8)) {
+        // Three and four token blocks, and two token blocks when eight waves are asked for: the activations of a
+        // window of WK k tiles are staged once per workgroup in LDS and shared by all its row groups (up to eight
+        // waves, one k tile of the window each; the two windows and the fold take up to 128 KiB of LDS).  Eight
+        // waves sharing one window beat two waves that gather their own activations at two token blocks
+        // (11008 x 4096, 32 tokens: 17.4 against 19.3 us) and four waves at four token blocks (64 tokens: 20.8
+        // against 22.4 us); sixteen waves lose again (18.6 us at 32 tokens), and at one token block the gather
+        // wins (15.9 against 16.4 us).
+        while (q.WK > 8) q.WK >>= 1;
         const int tiles_total = q.K / 32;
+        while (q.WK >= 2 && tiles_total % q.WK != 0) q.WK >>= 1;
         const size_t win_bytes = (size_t)2 * q.WK * CB * 68 * 16;
         size_t lds = (size_t)q.WK * RMAX * CB * 1024;
         if (win_bytes > lds) lds = win_bytes;
-        if (q.WK < 2 || tiles_total % q.WK != 0 || lds > 64 * 1024) return 1;      // does not apply: the caller falls back
-        gemm_wave_balanced_kernel<T, CB, RMAX, 2, true><<<wgs, q.WK * 64, lds, s>>>(q);
-        MLK_LAUNCH_CHECK();
-        return MLK_OK;
+        if (q.WK < 2 || lds > 150 * 1024) return 1;      // does not apply: the caller falls back
+        if constexpr (CB >= 2) {
+            // more than 64 KiB of dynamic LDS has to be allowed once per kernel and device
+            static bool ready_on[64] = {};
+            int dev = 0;
+            if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+            if (!ready_on[dev & 63]) {
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wave_balanced_kernel<T, CB, RMAX, 2, true>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+                if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));
+                ready_on[dev & 63] = true;
+            }
+            gemm_wave_balanced_kernel<T, CB, RMAX, 2, true><<<wgs, q.WK * 64, lds, s>>>(q);
+            MLK_LAUNCH_CHECK();
+            return MLK_OK;
+        }
     }
     while (q.WK * 64 > wave_kernel_threads(RMAX * CB, U, false) || (size_t)q.WK * RMAX * CB * 1024 > 64 * 1024) q.WK >>= 1;
     size_t lds = q.WK > 1 ? (size_t)q.WK * RMAX * CB * 1024 : 0;

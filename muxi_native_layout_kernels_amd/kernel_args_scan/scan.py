@@ -175,9 +175,9 @@ def scan_gemm(table, shapes, tokens, iters, progress=None):
             if m <= 16 and mode in ("rowmajor", "fp8"):
                 grid += [(10 + u, r, w, sk) for (_, r, w, sk) in list(grid) if _ == 1 for u in (2, 4, 6, 8)]
             # kernel 4: one workgroup per CU, row groups dealt out evenly (16-bit weights, up to 64 tokens; from three
-            # token blocks on with the activations shared through LDS and at most four waves)
+            # token blocks on, and at two token blocks with eight waves, the activations are shared through LDS)
             if mode == "rowmajor" and m <= 64:
-                grid += [(4, 1, w, 1) for w in ((1, 2, 4, 8) if m <= 32 else (2, 4))]
+                grid += [(4, 1, w, 1) for w in ((1, 2, 4, 8) if m <= 32 else (2, 4, 8))]
             # kernel 3: panels of 128 / 256 rows x 128 / 256 tokens (row-major operands, K % 128 == 0); above 64 tokens the
             # wave kernel is out of the race
             if mode in ("rowmajor", "fp8") and m > 64 and k % 128 == 0:

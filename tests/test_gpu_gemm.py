@@ -223,9 +223,9 @@ def test_gemm_balanced_rows_kernel(mlk, n, m):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("k", [192, 1024, 1152, 4096])
-@pytest.mark.parametrize("m", [33, 48, 50, 64])
+@pytest.mark.parametrize("m", [20, 32, 33, 48, 50, 64])
 def test_gemm_balanced_rows_kernel_shared_windows(mlk, dtype, k, m):
-    """kernelId 4 at three and four token blocks over short and long K: K = 192 (six k tiles, no whole
+    """kernelId 4 at two (eight waves), three and four token blocks over short and long K: K = 192 (six k tiles, no whole
     windows: the plain wave kernel takes it), 1024 and 4096 (the unrolled loop with its lead-in), 1152 (36 k
     tiles: nine windows, an odd tail), on 688 row groups (three and two per workgroup on 256 CUs); twice, and the
     two runs must agree bit for bit."""
@@ -234,7 +234,7 @@ def test_gemm_balanced_rows_kernel_shared_windows(mlk, dtype, k, m):
     b = randn((m, k), dtype, 1.0, 75)
     bias = randn((1, n), dtype, 1.0, 76)
     a = pack_a(w).cuda()
-    for p2 in (4, 2):
+    for p2 in (8, 4, 2):
         c = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=1, kernelParam2=p2, kernelParam3=1,
                                     kernelId=4, bias=bias.cuda())
         assert_close(c, ogemm.linear_expected(w, b, 0.5, bias), RTOL, ATOL, "balanced shared k=%d m=%d p2=%d" % (k, m, p2))
