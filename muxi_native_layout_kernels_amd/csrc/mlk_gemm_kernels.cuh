@@ -487,20 +487,37 @@ static int launch(const GemmArgs &p, hipStream_t s) {
     constexpr int U = (R * CB >= 8) ? 2 : ((R * CB >= 4) ? 3 : 4);
     GemmArgs q = p;
     while (q.WK * 64 > max_threads_for_tiles(R * CB) || (size_t)q.WK * R * CB * 1024 > 64 * 1024) q.WK >>= 1;
-    int row_tiles = (q.N / 16) / R;
-    int grid = row_tiles * q.SK;
+    auto grid_of = [](const GemmArgs &g) { return (g.N / 16) / R * g.SK; };
+    int grid = grid_of(q);
     size_t lds = q.WK > 1 ? (size_t)q.WK * R * CB * 1024 : 0;
     if constexpr (BMODE == MLK_B_ROWMAJOR && CB >= 2) {
         // stage row-major activations through LDS when every K slice is a whole number of WK-tile windows
-        const int tiles_total = q.K / 32;
-        const int tiles_per = (tiles_total + q.SK - 1) / q.SK;
-        const size_t win_bytes = (size_t)2 * q.WK * CB * 68 * 16;
         // (measured: staging pays from three token blocks up, and at two token blocks with eight waves to share a
-        // window; below that the direct gather wins)
-        if (g_tunable[1] && (CB >= 3 || q.WK >= 8) && q.WK >= 2 && tiles_total % q.SK == 0 && tiles_per % q.WK == 0 && win_bytes <= 48 * 1024) {
+        // window; below that the direct gather wins).  Up to eight waves share a window; the two windows and the
+        // fold may then need more than the 64 KiB a kernel gets without asking.
+        GemmArgs st = p;
+        while (st.WK > 8 || st.WK * 64 > max_threads_for_tiles(R * CB)) st.WK >>= 1;
+        const int tiles_total = st.K / 32;
+        const int tiles_per = (tiles_total + st.SK - 1) / st.SK;
+        const size_t win_bytes = (size_t)2 * st.WK * CB * 68 * 16;
+        size_t lds_st = (size_t)st.WK * R * CB * 1024;
+        if (win_bytes > lds_st) lds_st = win_bytes;
+        if (g_tunable[1] && (CB >= 3 || st.WK >= 8) && st.WK >= 2 && tiles_total % st.SK == 0 && tiles_per % st.WK == 0 &&
+            lds_st <= 150 * 1024) {
             constexpr int US = (R * CB >= 8) ? 2 : 4;
-            if (win_bytes > lds) lds = win_bytes;
-            gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, US, true><<<grid, q.WK * 64, lds, s>>>(q);
+            if (lds_st > 48 * 1024) {
+                static bool ready_on[64] = {};
+                int dev = 0;
+                if (hipGetDevice(&dev) != hipSuccess) dev = 0;
+                if (!ready_on[dev & 63]) {
+                    hipError_t e = hipFuncSetAttribute(
+                        reinterpret_cast<const void *>(&gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, US, true>),
+                        hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+                    if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));
+                    ready_on[dev & 63] = true;
+                }
+            }
+            gemm_wave_kernel<T, FP8, CB, R, BMODE, CMODE, US, true><<<grid_of(st), st.WK * 64, lds_st, s>>>(st);
             MLK_LAUNCH_CHECK();
             return MLK_OK;
         }
