@@ -48,6 +48,9 @@ struct GemmArgs {
     float alpha;
 };
 
+// Granules (16 bytes) between the activation fragments of neighbouring k tiles in a staged window.
+__host__ __device__ constexpr int stage_win_stride(int cb) { return cb * 68 + (cb % 2 == 0 ? 4 : 0); }
+
 // Threads per workgroup the wave kernel is compiled for: deep register rings (many tiles x many
 // k tiles in flight) get the register budget of a 256-thread workgroup instead of spilling.
 __host__ __device__ constexpr int wave_kernel_threads(int ntile, int depth, bool staged) {
@@ -130,9 +133,13 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
         // activations with row-contiguous 16-byte loads (WK*64 bytes per token), one step
         // ahead, and leaves them in LDS in MFMA fragment order (two buffers, one barrier per
         // step); each wave then reads its own tile's fragments with ds_read_b128.  Fragment
-        // rows are padded (68 granules per tile, 17 per k-octet) against bank conflicts.
+        // rows are padded (68 granules per tile, 17 per k-octet) against bank conflicts, and the fragments of
+        // neighbouring k tiles start 4 modulo 8 granules apart (stage_win_stride): a staging store puts the pieces
+        // of two neighbouring k tiles of one token row side by side in a group of eight lanes, and the banks
+        // repeat every 8 granules.
         u32x4 *win = reinterpret_cast<u32x4 *>(red);
-        const int win_granules = p.WK * CB * 68;
+        constexpr int WS = stage_win_stride(CB);
+        const int win_granules = p.WK * WS;
         const int nwin = (tend - tbeg) / p.WK;            // exact: the host only stages when WK divides the slice
         const int cols = p.WK * 4;                        // 16-byte granules per token in a window
         const int sh = __builtin_ctz(cols);
@@ -159,7 +166,7 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
             for (int i = 0; i < CB; ++i) {
                 const int g = threadIdx.x + i * blockDim.x;
                 const int row = g >> sh, colg = g & (cols - 1);
-                win[buf * win_granules + ((colg >> 2) * CB + (row >> 4)) * 68 + (colg & 3) * 17 + (row & 15)] = breg[i];
+                win[buf * win_granules + (colg >> 2) * WS + (row >> 4) * 68 + (colg & 3) * 17 + (row & 15)] = breg[i];
             }
         };
         auto issue_a = [&](int slot) {
@@ -173,7 +180,7 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
             if (do_stage) stage_load();
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = win[buf * win_granules + (wave * CB + cb) * 68 + q * 17 + r16];
+            for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = win[buf * win_granules + wave * WS + cb * 68 + q * 17 + r16];
             consume(slot);
             if (do_issue) issue_a(slot);
             __builtin_amdgcn_sched_barrier(0);
@@ -499,7 +506,7 @@ static int launch(const GemmArgs &p, hipStream_t s) {
         while (st.WK > 8 || st.WK * 64 > max_threads_for_tiles(R * CB)) st.WK >>= 1;
         const int tiles_total = st.K / 32;
         const int tiles_per = (tiles_total + st.SK - 1) / st.SK;
-        const size_t win_bytes = (size_t)2 * st.WK * CB * 68 * 16;
+        const size_t win_bytes = (size_t)2 * st.WK * stage_win_stride(CB) * 16;
         size_t lds_st = (size_t)st.WK * R * CB * 1024;
         if (win_bytes > lds_st) lds_st = win_bytes;
         if (g_tunable[1] && (CB >= 3 || st.WK >= 8) && st.WK >= 2 && tiles_total % st.SK == 0 && tiles_per % st.WK == 0 &&
@@ -559,7 +566,7 @@ static int launch_balanced(const GemmArgs &p, int wgs, hipStream_t s) {
         while (q.WK > 8) q.WK >>= 1;
         const int tiles_total = q.K / 32;
         while (q.WK >= 2 && tiles_total % q.WK != 0) q.WK >>= 1;
-        const size_t win_bytes = (size_t)2 * q.WK * CB * 68 * 16;
+        const size_t win_bytes = (size_t)2 * q.WK * stage_win_stride(CB) * 16;
         size_t lds = (size_t)q.WK * RMAX * CB * 1024;
         if (win_bytes > lds) lds = win_bytes;
         if (q.WK < 2 || lds > 150 * 1024) return 1;      // does not apply: the caller falls back
