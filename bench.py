@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the native-layout hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--case TEXT] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--case TEXT] [--no-cpu] [--case-steps S]
 
 Prints ONE JSON line.  The headline workload is the fp16 narrow GeMM of the
 second benchmark configuration (`gemm_layoutA`, weights 11008 x 4096 in
@@ -11,12 +11,18 @@ different weight copy (enough copies to exceed the 256 MiB Infinity Cache), so
 the bandwidth is HBM bandwidth.
 
 Timing protocol: the K calls are recorded into one HIP graph.  After the W
-warm-up calls and un-timed replays of the graph for at least 20 ms (the capture
+warm-up calls and un-timed replays of the graph for at least 100 ms, the graph
+is replayed five times, each replay (exactly K calls) bracketed by HIP events
+on the stream that runs it.  The headline value comes from the first timed
+replay; the median and the minimum of the five are reported beside it, and
+for every other configuration.  Why 100 ms and why long replays: the capture
 leaves the GPU idle and the first replays after an idle period run several
-percent below the steady state), the graph is replayed five times, each replay
-(exactly K calls) bracketed by HIP events on the stream that runs it.  The
-headline value comes from the first timed replay; the median and the minimum
-of the five are reported beside it, and for every other configuration.
+percent below the steady state; the kernels that stream the largest matrices
+(the 235 MB soft-FP8 GeMV / GeMM) only reach their steady state after some
+50 to 100 ms of continuous load (38.4 us per call in 4 ms replays after 40 ms,
+36.3 us in 38 ms replays after 100 ms).  The GeMV / GeMM configurations
+therefore time 1000 calls per replay (--case-steps), as the reference's own
+benchmark scripts time long back-to-back runs.
 
 `per_config` holds the other configurations (bf16 / soft-FP8 GeMV, the M sweep,
 the native-layout chain, the relayout kernels and the fused MoE layer) with
@@ -47,9 +53,12 @@ TIMED_REPLAYS = 5
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--steps", type=int, default=1000)
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--quick", action="store_true", help="headline workload only")
+    ap.add_argument("--moe-steps", type=int, default=20, help="fused_moe calls per timed replay")
+    ap.add_argument("--case-steps", type=int, default=1000,
+                    help="calls per timed replay of the per-configuration cases (never more than --steps)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
     ap.add_argument("--case", default=None,
                     help="besides the headline, run only the per-configuration cases whose name contains this text "
@@ -101,7 +110,7 @@ def main():
     bench_stream = torch.cuda.Stream()      # every timed region runs on this one stream
 
     def settle_replays(steps):
-        return 1 + max(1, int(0.02 / (steps * 20e-6)))      # >= 20 ms at 20 us per call
+        return 1 + max(1, int(0.1 / (steps * 20e-6)))       # >= 100 ms at 20 us per call
 
     def run_graph(calls, steps, warmup, reps=TIMED_REPLAYS):
         """Replay `steps` calls (cycling through `calls`) from one HIP graph, `reps` times, each replay between
@@ -251,7 +260,7 @@ def main():
         extra = dict(params=[block, kid, p1, p2], copies=len(A))
         del A
         if yardstick:
-            extra["read_only_us"] = read_only_us(wbytes, min(steps, 60))
+            extra["read_only_us"] = read_only_us(wbytes, steps)
         extra["cpu_baseline"] = cpu_linear(n, k, 1, kind, cpu_rows)
         return finish(name, t, algo, **extra)
 
@@ -306,7 +315,7 @@ def main():
         if blas and kind != 2:
             count = len(A)
             del A
-            blas_yardstick(row, n, k, DT[kind], m, min(steps, 100), count)
+            blas_yardstick(row, n, k, DT[kind], m, steps, count)
         return row
 
     def panel_case(name, n, k, kind, m, steps):
@@ -488,8 +497,8 @@ def main():
                             "the Infinity Cache, not HBM; reported for information, never the headline"}
         ceiling = round(read_ceiling(40), 1)
         # the same yardstick at the headline's size: one launch that only reads as many bytes as the weights hold
-        same_size = read_only_us(N * K_ * 2, min(args.steps, 100))
-        short = max(20, min(args.steps, 100))
+        same_size = read_only_us(N * K_ * 2, args.steps)
+        short = max(20, min(args.steps, args.case_steps))
         add(gemv_case, "C1 bf16 gemv 4096x4096", 4096, 4096, 1, short, 10, yardstick=True, cpu_rows=4096)
         for m in (1, 8, 32, 64):
             add(gemm_case, "C2 fp16 gemm_layoutA 11008x4096 M=%d" % m, N, K_, 0, m, short, 10, blas=True)
@@ -503,11 +512,11 @@ def main():
         add(relayout_case, "C4 reLayoutC bf16 [32, 8192]", "reLayoutC", short)
         add(relayout_case, "C3 fp8_weight_repack 28672x8192", "fp8_weight_repack", 10)
         for T in (1, 16, 64, 256):
-            add(moe_case, "C5 bf16 fused_moe T=%d" % T, T, False, 20, 5)
+            add(moe_case, "C5 bf16 fused_moe T=%d" % T, T, False, args.moe_steps, 5)
         for T in (1, 16, 64, 256):
-            add(moe_case, "C5 soft-fp8 fused_moe T=%d" % T, T, True, 20, 5)
+            add(moe_case, "C5 soft-fp8 fused_moe T=%d" % T, T, True, args.moe_steps, 5)
         for T in (1, 16):
-            add(moe_next_case, "next: grouped-routing MoE E=256 top-8 H=7168 I=2048 bf16 T=%d" % T, T, 20, 5)
+            add(moe_next_case, "next: grouped-routing MoE E=256 top-8 H=7168 I=2048 bf16 T=%d" % T, T, args.moe_steps, 5)
         moe_w.clear()
         torch.cuda.empty_cache()
         for m in (128, 256, 1024, 4096):
