@@ -59,7 +59,7 @@ __host__ __device__ constexpr int wave_kernel_threads(int ntile, int depth, bool
 
 // The body of the wave kernel for the R row groups from rg0 (row tile rt of `row_tiles`, K slice sk).
 // red: [WK][R*CB][64] f32x4 of LDS; the staged variant first uses it for two activation windows.
-template <class T, bool FP8, int CB, int R, int BMODE, int CMODE, int U, bool STAGE>
+template <class T, bool FP8, int CB, int R, int BMODE, int CMODE, int U, bool STAGE, bool TWOSC = false>
 __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, const int sk, const int rg0,
                                                const int row_tiles, f32x4 *red, int &s_last) {
     const int lane = threadIdx.x & 63;
@@ -92,9 +92,16 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
     }
     const size_t bstep = (BMODE == MLK_B_NATIVE) ? (size_t)mb_total * 512 : 32;  // elements per k tile
 
-    // the R row groups of a wave (R divides 8, rg0 is a multiple of R) share one row of block scales
-    ScaleRow srow;
+    // The R row groups of a wave share one row of block scales (R divides 8, rg0 is a multiple of R).  TWOSC: rg0
+    // is arbitrary and R <= 8, so the row groups may lie in two neighbouring 128-row blocks: the first `split` of
+    // them take the scales of the first block, the others those of the second.
+    ScaleRow srow, srow2;
+    int split = R;
     if (FP8) srow = load_scale_row(p.scale ? p.scale + (size_t)(rg0 >> 3) * scale_cols : nullptr, scale_cols, lane);
+    if (FP8 && TWOSC) {
+        split = 8 - (rg0 & 7);
+        srow2 = load_scale_row(p.scale ? p.scale + (size_t)((rg0 + R - 1) >> 3) * scale_cols : nullptr, scale_cols, lane);
+    }
 
     f32x4 acc[R][CB];
 #pragma unroll
@@ -107,10 +114,12 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
     WeightFrag<FP8> wf[U][R];
     u32x4 bf[U][CB];
     float sc[U];        // one block scale per k tile: the R row groups of a wave share a 128-row block
+    float sc2[U];       // TWOSC: the scale of the second block
     auto issue = [&](int slot, int kt) {
 #pragma unroll
         for (int r = 0; r < R; ++r) wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
         if (FP8) sc[slot] = scale_at(srow, kt >> 2);
+        if (FP8 && TWOSC) sc2[slot] = scale_at(srow2, kt >> 2);
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) bf[slot][cb] = ld_global_u32x4(bptr[cb] + (size_t)kt * bstep);
     };
@@ -118,7 +127,7 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
         u32x4 a[R], b[CB];
         float sv[R];
 #pragma unroll
-        for (int r = 0; r < R; ++r) sv[r] = FP8 ? sc[slot] : 1.f;
+        for (int r = 0; r < R; ++r) sv[r] = FP8 ? ((TWOSC && r >= split) ? sc2[slot] : sc[slot]) : 1.f;
         weight_operands<FP8, R>(a, wf[slot], sv);
 #pragma unroll
         for (int cb = 0; cb < CB; ++cb) b[cb] = bf[slot][cb];
@@ -174,6 +183,7 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
 #pragma unroll
             for (int r = 0; r < R; ++r) wf[slot][r] = load_weight_frag<FP8>(abase[r], kt, lane);
             if (FP8) sc[slot] = scale_at(srow, kt >> 2);
+            if (FP8 && TWOSC) sc2[slot] = scale_at(srow2, kt >> 2);
         };
         auto step = [&](int slot, int buf, bool do_stage, bool do_issue) {
             // pinned ahead of the products: the compiler would sink these loads to the parking stores below
@@ -355,7 +365,7 @@ __global__ void __launch_bounds__(wave_kernel_threads(R *CB, U, STAGE)) gemm_wav
 // fully unrolled body; the test is uniform for the workgroup.  Row-major operands, no K split.  STAGE: the
 // activations of a window of WK k tiles are fetched once per workgroup and shared by all its row groups through
 // LDS (three and four token blocks).
-template <class T, int CB, int RMAX, int U, bool STAGE = false>
+template <class T, int CB, int RMAX, int U, bool STAGE = false, bool FP8 = false>
 __global__ void __launch_bounds__(STAGE ? 512 : wave_kernel_threads(RMAX *CB, U, STAGE)) gemm_wave_balanced_kernel(GemmArgs p) {
     extern __shared__ f32x4 red[];
     __shared__ int s_last;
@@ -363,10 +373,11 @@ __global__ void __launch_bounds__(STAGE ? 512 : wave_kernel_threads(RMAX *CB, U,
     const int rt = blockIdx.x;
     const int rg0 = (int)((long long)rt * groups / (int)gridDim.x);
     const int nr = (int)((long long)(rt + 1) * groups / (int)gridDim.x) - rg0;
+    // soft-FP8: a workgroup's row groups start anywhere, so they may straddle two 128-row blocks of scales
     if (nr == RMAX)
-        gemm_wave_body<T, false, CB, RMAX, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR, U, STAGE>(p, rt, 0, rg0, gridDim.x, red, s_last);
+        gemm_wave_body<T, FP8, CB, RMAX, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR, U, STAGE, FP8>(p, rt, 0, rg0, gridDim.x, red, s_last);
     else
-        gemm_wave_body<T, false, CB, RMAX - 1, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR, U, STAGE>(p, rt, 0, rg0, gridDim.x, red, s_last);
+        gemm_wave_body<T, FP8, CB, RMAX - 1, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR, U, STAGE, FP8>(p, rt, 0, rg0, gridDim.x, red, s_last);
 }
 
 // Kernel 2: row-shared tile kernel (see mlk_tile.cuh).  Four waves per workgroup, R row groups
@@ -550,7 +561,7 @@ static int launch(const GemmArgs &p, hipStream_t s) {
 // few rows: with a fixed number of row groups per workgroup the grid of N = 11008 at 16 tokens is 172
 // workgroups, a third of the CUs idle and the others over their share.  Kernel id 4 runs one workgroup
 // per CU instead.
-template <class T, int CB, int RMAX>
+template <class T, int CB, int RMAX, bool FP8 = false>
 static int launch_balanced(const GemmArgs &p, int wgs, hipStream_t s) {
     constexpr int U = RMAX * CB <= 4 ? 4 : (RMAX * CB <= 8 ? 3 : 2);     // k tiles in flight per wave
     GemmArgs q = p;
@@ -576,16 +587,17 @@ static int launch_balanced(const GemmArgs &p, int wgs, hipStream_t s) {
             int dev = 0;
             if (hipGetDevice(&dev) != hipSuccess) dev = 0;
             if (!ready_on[dev & 63]) {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wave_balanced_kernel<T, CB, RMAX, 2, true>),
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wave_balanced_kernel<T, CB, RMAX, 2, true, FP8>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
                 if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));
                 ready_on[dev & 63] = true;
             }
-            gemm_wave_balanced_kernel<T, CB, RMAX, 2, true><<<wgs, q.WK * 64, lds, s>>>(q);
+            gemm_wave_balanced_kernel<T, CB, RMAX, 2, true, FP8><<<wgs, q.WK * 64, lds, s>>>(q);
             MLK_LAUNCH_CHECK();
             return MLK_OK;
         }
     }
+    if constexpr (FP8) return 1;     // soft-FP8 weights take this kernel only with staged windows
     while (q.WK * 64 > wave_kernel_threads(RMAX * CB, U, false) || (size_t)q.WK * RMAX * CB * 1024 > 64 * 1024) q.WK >>= 1;
     size_t lds = q.WK > 1 ? (size_t)q.WK * RMAX * CB * 1024 : 0;
     gemm_wave_balanced_kernel<T, CB, RMAX, U><<<wgs, q.WK * 64, lds, s>>>(q);
@@ -610,6 +622,21 @@ static int launch_rc(const GemmArgs &p, int kernel_id, int R, int CB, hipStream_
     if (R == RR && CB == CC)                                                                    \
         return (kernel_id == 2 && tile_kernel_fits(p, RR, CC)) ? launch_tile<T, FP8, CC, RR, BMODE, CMODE>(p, s) \
                                                           : launch<T, FP8, CC, RR, BMODE, CMODE>(p, s);
+    if constexpr (FP8 && BMODE == MLK_B_ROWMAJOR && CMODE == MLK_C_ROWMAJOR) {
+        if (kernel_id == 4 && CB >= 2) {
+            int r_max = 0;
+            const int wgs = p.SK == 1 ? balanced_grid(p, CB, &r_max) : 0;
+#define MLK_BAL8(CC, RR)                                                  \
+    if (wgs && CB == CC && r_max == RR) {                                 \
+        const int rc = launch_balanced<T, CC, RR, true>(p, wgs, s);       \
+        if (rc <= 0) return rc;                                           \
+    }
+            MLK_BAL8(2, 2) MLK_BAL8(2, 3) MLK_BAL8(2, 4)
+            MLK_BAL8(3, 2) MLK_BAL8(3, 3) MLK_BAL8(3, 4)
+            MLK_BAL8(4, 2) MLK_BAL8(4, 3) MLK_BAL8(4, 4)
+#undef MLK_BAL8
+        }
+    }
     if constexpr (!FP8 && BMODE == MLK_B_ROWMAJOR && CMODE == MLK_C_ROWMAJOR) {
         if (kernel_id == 4) {
             int r_max = 0;

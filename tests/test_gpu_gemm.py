@@ -243,8 +243,27 @@ def test_gemm_balanced_rows_kernel_shared_windows(mlk, dtype, k, m):
         assert torch.equal(c, c2)
 
 
+@pytest.mark.parametrize("n", [11008, 12288, 4736])
+@pytest.mark.parametrize("m", [20, 32, 40, 64])
+def test_gemm_balanced_rows_kernel_soft_fp8(mlk, n, m):
+    """kernelId 4 with soft-FP8 weights from two token blocks on (eight waves share staged windows): three or two
+    row groups per workgroup that start anywhere, so they straddle two 128-row blocks of scales; every block has
+    its own random scale.  With two waves at two token blocks the id means kernel 1."""
+    k = 1024
+    codes = fp8_codes((n, k), 91)
+    g = torch.Generator().manual_seed(92)
+    scale = (torch.rand((n // 128, k // 128), generator=g) * 0.02 + 0.001).float()
+    b = randn((m, k), torch.bfloat16, 1.0, 93)
+    a = pack_a(codes).cuda()
+    want = ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), b)
+    for p2 in (8, 4, 2):
+        c = mlk.gemm_layoutA_soft_fp8_wapper(a, scale.cuda(), b.cuda(), n, m, k, kernelParam1=1, kernelParam2=p2,
+                                             kernelParam3=1, kernelId=4)
+        assert_close(c, want, RTOL, ATOL, "balanced fp8 n=%d m=%d p2=%d" % (n, m, p2))
+
+
 def test_gemm_balanced_rows_fallbacks(mlk):
-    """Soft-FP8 weights and native operands are outside kernel 4: the id then means kernel 1."""
+    """Soft-FP8 weights at one token block and native operands are outside kernel 4: the id then means kernel 1."""
     n, k, m = 16 * 300, 512, 16
     codes = fp8_codes((n - n % 128, k), 81)
     n8 = codes.shape[0]
