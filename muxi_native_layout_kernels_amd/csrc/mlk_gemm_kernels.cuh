@@ -165,17 +165,28 @@ __device__ __forceinline__ void gemm_wave_body(const GemmArgs &p, const int rt, 
 #pragma unroll
             for (int i = 0; i < CB; ++i) {
                 const int g = threadIdx.x + i * blockDim.x;
-                const int row = g >> sh, colg = g & (cols - 1);
-                const int tok = min(p.cb0 * 16 + row, p.M_total - 1);
-                breg[i] = ld_global_u32x4(p.B + (size_t)tok * p.K + (size_t)tile0 * 32 + colg * 8);
+                if constexpr (BMODE == MLK_B_NATIVE) {
+                    // layout-B: the fragment of (k tile, token block) is 1 KiB in one piece, already in MFMA order
+                    const int f = g >> 6, w = f / CB, cb = f - w * CB;
+                    breg[i] = ld_global_u32x4(p.B + (((size_t)(tile0 + w) * mb_total + p.cb0 + cb) * 64 + (g & 63)) * 8);
+                } else {
+                    const int row = g >> sh, colg = g & (cols - 1);
+                    const int tok = min(p.cb0 * 16 + row, p.M_total - 1);
+                    breg[i] = ld_global_u32x4(p.B + (size_t)tok * p.K + (size_t)tile0 * 32 + colg * 8);
+                }
             }
         };
         auto stage_store = [&](int buf) {
 #pragma unroll
             for (int i = 0; i < CB; ++i) {
                 const int g = threadIdx.x + i * blockDim.x;
-                const int row = g >> sh, colg = g & (cols - 1);
-                win[buf * win_granules + (colg >> 2) * WS + (row >> 4) * 68 + (colg & 3) * 17 + (row & 15)] = breg[i];
+                if constexpr (BMODE == MLK_B_NATIVE) {
+                    const int f = g >> 6, w = f / CB, cb = f - w * CB, j = g & 63;
+                    win[buf * win_granules + w * WS + cb * 68 + (j >> 4) * 17 + (j & 15)] = breg[i];
+                } else {
+                    const int row = g >> sh, colg = g & (cols - 1);
+                    win[buf * win_granules + (colg >> 2) * WS + (row >> 4) * 68 + (colg & 3) * 17 + (row & 15)] = breg[i];
+                }
             }
         };
         auto issue_a = [&](int slot) {
@@ -365,7 +376,8 @@ __global__ void __launch_bounds__(wave_kernel_threads(R *CB, U, STAGE)) gemm_wav
 // fully unrolled body; the test is uniform for the workgroup.  Row-major operands, no K split.  STAGE: the
 // activations of a window of WK k tiles are fetched once per workgroup and shared by all its row groups through
 // LDS (three and four token blocks).
-template <class T, int CB, int RMAX, int U, bool STAGE = false, bool FP8 = false>
+template <class T, int CB, int RMAX, int U, bool STAGE = false, bool FP8 = false, int BMODE = MLK_B_ROWMAJOR,
+          int CMODE = MLK_C_ROWMAJOR>
 __global__ void __launch_bounds__(STAGE ? 512 : wave_kernel_threads(RMAX *CB, U, STAGE)) gemm_wave_balanced_kernel(GemmArgs p) {
     extern __shared__ f32x4 red[];
     __shared__ int s_last;
@@ -375,9 +387,9 @@ __global__ void __launch_bounds__(STAGE ? 512 : wave_kernel_threads(RMAX *CB, U,
     const int nr = (int)((long long)(rt + 1) * groups / (int)gridDim.x) - rg0;
     // soft-FP8: a workgroup's row groups start anywhere, so they may straddle two 128-row blocks of scales
     if (nr == RMAX)
-        gemm_wave_body<T, FP8, CB, RMAX, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR, U, STAGE, FP8>(p, rt, 0, rg0, gridDim.x, red, s_last);
+        gemm_wave_body<T, FP8, CB, RMAX, BMODE, CMODE, U, STAGE, FP8>(p, rt, 0, rg0, gridDim.x, red, s_last);
     else
-        gemm_wave_body<T, FP8, CB, RMAX - 1, MLK_B_ROWMAJOR, MLK_C_ROWMAJOR, U, STAGE, FP8>(p, rt, 0, rg0, gridDim.x, red, s_last);
+        gemm_wave_body<T, FP8, CB, RMAX - 1, BMODE, CMODE, U, STAGE, FP8>(p, rt, 0, rg0, gridDim.x, red, s_last);
 }
 
 // Kernel 2: row-shared tile kernel (see mlk_tile.cuh).  Four waves per workgroup, R row groups
@@ -561,7 +573,7 @@ static int launch(const GemmArgs &p, hipStream_t s) {
 // few rows: with a fixed number of row groups per workgroup the grid of N = 11008 at 16 tokens is 172
 // workgroups, a third of the CUs idle and the others over their share.  Kernel id 4 runs one workgroup
 // per CU instead.
-template <class T, int CB, int RMAX, bool FP8 = false>
+template <class T, int CB, int RMAX, bool FP8 = false, int BMODE = MLK_B_ROWMAJOR, int CMODE = MLK_C_ROWMAJOR>
 static int launch_balanced(const GemmArgs &p, int wgs, hipStream_t s) {
     constexpr int U = RMAX * CB <= 4 ? 4 : (RMAX * CB <= 8 ? 3 : 2);     // k tiles in flight per wave
     GemmArgs q = p;
@@ -587,17 +599,18 @@ static int launch_balanced(const GemmArgs &p, int wgs, hipStream_t s) {
             int dev = 0;
             if (hipGetDevice(&dev) != hipSuccess) dev = 0;
             if (!ready_on[dev & 63]) {
-                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wave_balanced_kernel<T, CB, RMAX, 2, true, FP8>),
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_wave_balanced_kernel<T, CB, RMAX, 2, true, FP8, BMODE, CMODE>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
                 if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));
                 ready_on[dev & 63] = true;
             }
-            gemm_wave_balanced_kernel<T, CB, RMAX, 2, true, FP8><<<wgs, q.WK * 64, lds, s>>>(q);
+            gemm_wave_balanced_kernel<T, CB, RMAX, 2, true, FP8, BMODE, CMODE><<<wgs, q.WK * 64, lds, s>>>(q);
             MLK_LAUNCH_CHECK();
             return MLK_OK;
         }
     }
-    if constexpr (FP8) return 1;     // soft-FP8 weights take this kernel only with staged windows
+    // soft-FP8 weights and layout-B activations take this kernel only with staged windows
+    if constexpr (FP8 || BMODE != MLK_B_ROWMAJOR) return 1;
     while (q.WK * 64 > wave_kernel_threads(RMAX * CB, U, false) || (size_t)q.WK * RMAX * CB * 1024 > 64 * 1024) q.WK >>= 1;
     size_t lds = q.WK > 1 ? (size_t)q.WK * RMAX * CB * 1024 : 0;
     gemm_wave_balanced_kernel<T, CB, RMAX, U><<<wgs, q.WK * 64, lds, s>>>(q);
@@ -622,6 +635,22 @@ static int launch_rc(const GemmArgs &p, int kernel_id, int R, int CB, hipStream_
     if (R == RR && CB == CC)                                                                    \
         return (kernel_id == 2 && tile_kernel_fits(p, RR, CC)) ? launch_tile<T, FP8, CC, RR, BMODE, CMODE>(p, s) \
                                                           : launch<T, FP8, CC, RR, BMODE, CMODE>(p, s);
+    if constexpr (!FP8 && BMODE == MLK_B_NATIVE) {
+        // layout-B activations (row-major or layout-C output): kernel id 4 from two token blocks on, staged windows
+        if (kernel_id == 4 && CB >= 2) {
+            int r_max = 0;
+            const int wgs = p.SK == 1 ? balanced_grid(p, CB, &r_max) : 0;
+#define MLK_BALN(CC, RR)                                                                 \
+    if (wgs && CB == CC && r_max == RR) {                                                \
+        const int rc = launch_balanced<T, CC, RR, false, BMODE, CMODE>(p, wgs, s);       \
+        if (rc <= 0) return rc;                                                          \
+    }
+            MLK_BALN(2, 2) MLK_BALN(2, 3) MLK_BALN(2, 4)
+            MLK_BALN(3, 2) MLK_BALN(3, 3) MLK_BALN(3, 4)
+            MLK_BALN(4, 2) MLK_BALN(4, 3) MLK_BALN(4, 4)
+#undef MLK_BALN
+        }
+    }
     if constexpr (FP8 && BMODE == MLK_B_ROWMAJOR && CMODE == MLK_C_ROWMAJOR) {
         if (kernel_id == 4 && CB >= 2) {
             int r_max = 0;

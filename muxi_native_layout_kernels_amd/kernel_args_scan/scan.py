@@ -178,8 +178,8 @@ def scan_gemm(table, shapes, tokens, iters, progress=None):
             # token blocks on, and at two token blocks with eight waves, the activations are shared through LDS)
             if mode == "rowmajor" and m <= 64:
                 grid += [(4, 1, w, 1) for w in ((1, 2, 4, 8) if m <= 32 else (2, 4, 8))]
-            # the same with soft-FP8 weights, from two token blocks on (staged windows only)
-            if mode == "fp8" and 16 < m <= 64:
+            # the same with soft-FP8 weights or layout-B activations, from two token blocks on (staged windows only)
+            if mode in ("fp8", "continuous", "native") and 16 < m <= 64:
                 grid += [(4, 1, w, 1) for w in (4, 8)]
             # kernel 3: panels of 128 / 256 rows x 128 / 256 tokens (row-major operands, K % 128 == 0); above 64 tokens the
             # wave kernel is out of the race

@@ -292,6 +292,26 @@ def test_gemm_special_cases(mlk):
 
 
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("m", [32, 48, 64])
+def test_native_chain_balanced_rows_kernel(mlk, dtype, m):
+    """kernelId 4 on layout-B activations from two token blocks on (eight and four waves share staged windows):
+    layout-C output + reLayoutC equals the row-major output bit for bit, the layout-C tensor equals the oracle's
+    relayout of it, and both match the oracle; 688 and 512 row groups (three / two and two per workgroup)."""
+    for n, k in ((16 * 688, 1024), (8192, 512)):
+        w = randn((n, k), dtype, 0.02, 18)
+        b = randn((m, k), dtype, 1.0, 19)
+        a, b_nat = pack_a(w).cuda(), mlk.layoutB(b.cuda())
+        for p2 in (8, 4):
+            c_rm = mlk.gemm_layoutAB_ContinuousC_wapper(a, b_nat, n, m, k, kernelParam1=1, kernelParam2=p2, kernelParam3=1,
+                                                        kernelId=4)
+            c_nat = mlk.gemm_layoutABC_wapper(a, b_nat, n, m, k, kernelParam1=1, kernelParam2=p2, kernelParam3=1,
+                                              kernelId=4)
+            assert torch.equal(mlk.reLayoutC(c_nat), c_rm)
+            assert torch.equal(c_nat.cpu().view(torch.int16), ogemm.layout_c_of(c_rm.cpu()).view(torch.int16))
+            assert_close(c_rm, ogemm.linear_expected(w, b), RTOL, ATOL, "native balanced n=%d m=%d p2=%d" % (n, m, p2))
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_native_chain_bit_exact(mlk, dtype):
     """layoutB -> gemm_layoutABC -> reLayoutC equals gemm_layoutAB_ContinuousC bit for bit (same launch
     parameters, hence same accumulation order), and both match the oracle."""
