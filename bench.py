@@ -57,6 +57,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=50)
     ap.add_argument("--quick", action="store_true", help="headline workload only")
     ap.add_argument("--moe-steps", type=int, default=20, help="fused_moe calls per timed replay")
+    ap.add_argument("--no-blas", action="store_true", help="skip the vendor BLAS yardsticks (counter runs)")
     ap.add_argument("--case-steps", type=int, default=1000,
                     help="calls per timed replay of the per-configuration cases (never more than --steps)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline legs")
@@ -312,7 +313,7 @@ def main():
         row = finish(name, t, algo, params=[kid, p1, p2, p3], copies=len(A))
         if cpu:
             row["cpu_baseline"] = cpu_linear(n, k, m, kind, cpu_rows, native=native)
-        if blas and kind != 2:
+        if blas and kind != 2 and not args.no_blas:
             count = len(A)
             del A
             blas_yardstick(row, n, k, DT[kind], m, steps, count)
