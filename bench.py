@@ -13,9 +13,16 @@ the bandwidth is HBM bandwidth.
 Timing protocol: the K calls are recorded into one HIP graph.  After the W
 warm-up calls and un-timed replays of the graph for at least 100 ms, the graph
 is replayed five times, each replay (exactly K calls) bracketed by HIP events
-on the stream that runs it.  The headline value comes from the first timed
-replay; the median and the minimum of the five are reported beside it, and
-for every other configuration.  Why 100 ms and why long replays: the capture
+on the stream that runs it and queued behind at least half a millisecond of
+un-timed replays.  A graph takes some 7 us from its launch to its first kernel
+even then, and a short graph bills that to its few calls (+0.4 us per call at
+K = 20, +1.5 us at K = 5): below K = 200 the timed GeMV / GeMM calls are
+therefore launched one by one between the events, behind 5 ms of queued
+replays that give the host its head start (16.0 us per call at any K, against
+15.9 us from a graph of 1000).  The headline value comes from the first timed replay; the
+median and the minimum of the five are reported beside it, and for every
+other configuration.  `ms_per_step` is the host clock around one more replay
+between two synchronizations, launch latency included.  Why 100 ms and why long replays: the capture
 leaves the GPU idle and the first replays after an idle period run several
 percent below the steady state; the kernels that stream the largest matrices
 (the 235 MB soft-FP8 GeMV / GeMM) only reach their steady state after some
@@ -113,10 +120,15 @@ def main():
     def settle_replays(steps):
         return 1 + max(1, int(0.1 / (steps * 20e-6)))       # >= 100 ms at 20 us per call
 
-    def run_graph(calls, steps, warmup, reps=TIMED_REPLAYS):
-        """Replay `steps` calls (cycling through `calls`) from one HIP graph, `reps` times, each replay between
-        HIP events on the launching stream.  Returns microseconds per call of the first timed replay, the median
-        and the minimum over the replays, and the wall seconds of the first timed replay."""
+    def run_graph(calls, steps, warmup, reps=TIMED_REPLAYS, direct_if_short=False):
+        """Time `steps` calls (cycling through `calls`) `reps` times, each time between HIP events on the launching
+        stream and queued behind un-timed work, so that the first timed call starts on a busy GPU.  The timed calls
+        are one replay of a HIP graph that holds them.  A graph takes some 7 us from its launch to its first kernel
+        even when it is queued behind other work, which a short graph bills to its few calls; so with
+        `direct_if_short` (plain library calls, cheap on the host) fewer than 200 steps are launched one by one
+        instead, behind 5 ms of queued replays that give the host its head start.  Returns microseconds per call of
+        the first timed run, the median and the minimum over the runs, and the host-clock seconds of one more replay
+        of the graph between two synchronizations."""
         stream = bench_stream
         with torch.cuda.stream(stream):
             for i in range(max(warmup, 3)):
@@ -129,22 +141,36 @@ def main():
             for _ in range(settle_replays(steps)):
                 graph.replay()
             torch.cuda.synchronize()
-            us, wall = [], None
-            for _ in range(reps):
+
+            def timed(lead, direct):
                 e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-                t0 = time.perf_counter()
+                for _ in range(lead):
+                    graph.replay()
                 e0.record()
-                graph.replay()
+                if direct:
+                    for i in range(steps):
+                        calls[i % len(calls)]()
+                else:
+                    graph.replay()
                 e1.record()
                 torch.cuda.synchronize()
-                if wall is None:
-                    wall = time.perf_counter() - t0
-                us.append(e0.elapsed_time(e1) * 1e3 / steps)
-        return dict(us=us[0], us_median=statistics.median(us), us_min=min(us), wall=wall)
+                return e0.elapsed_time(e1) * 1e3 / steps
+
+            direct = direct_if_short and steps < 200
+            lead = max(1, -(-500 // (steps * 15)))           # >= 0.5 ms of un-timed replays ahead of a timed one
+            if direct:
+                lead = max(1, int(5000.0 / (steps * timed(lead, False))) + 1)
+            us = [timed(lead, direct) for _ in range(reps)]
+            t0 = time.perf_counter()
+            graph.replay()
+            torch.cuda.synchronize()
+            wall = time.perf_counter() - t0
+        return dict(us=us[0], us_median=statistics.median(us), us_min=min(us), wall=wall,
+                    how="launched one by one behind queued graph replays" if direct else "one graph replay")
 
     def finish(name, t, algo, **extra):
         row = dict(name=name, us=t["us"], us_median=t["us_median"], us_min=t["us_min"], bytes=algo,
-                   gbps=algo / t["us"] / 1e3, frac=algo / t["us"] / 1e3 / HBM_PEAK_GBPS, wall=t["wall"])
+                   gbps=algo / t["us"] / 1e3, frac=algo / t["us"] / 1e3 / HBM_PEAK_GBPS, wall=t["wall"], how=t["how"])
         row.update(extra)
         got = traffic_table.get(name)
         if isinstance(got, dict):   # counted for one routing: valid only when this run drew as many active experts
@@ -168,7 +194,7 @@ def main():
                     _lib.check(lib.mlk_stream_read(b.data_ptr(), nbytes, block, wgs, 0,
                                                    torch.cuda.current_stream().cuda_stream), "stream_read")
                 return call
-            t = run_graph([mk(b) for b in bufs], steps, 5, reps=3)
+            t = run_graph([mk(b) for b in bufs], steps, 5, reps=3, direct_if_short=True)
             best = t["us_median"] if best is None else min(best, t["us_median"])
         return best
 
@@ -256,7 +282,7 @@ def main():
                                                  0 if scale is None else scale.data_ptr(), block, kid, p1, p2, st),
                            "gemv")
             return call
-        t = run_graph([mk(a) for a in A], steps, warmup)
+        t = run_graph([mk(a) for a in A], steps, warmup, direct_if_short=True)
         algo = wbytes + (scale.numel() * 4 if scale is not None else 0) + k * 2 + n * 2
         extra = dict(params=[block, kid, p1, p2], copies=len(A))
         del A
@@ -270,7 +296,7 @@ def main():
         W = [(torch.randn((n, k), generator=gen, device=dev) * 0.02).to(dt) for _ in range(count)]
         b = torch.randn((m, k), generator=gen, device=dev).to(dt)
         out = torch.empty((m, n), dtype=dt, device=dev)
-        t = run_graph([(lambda w=w: torch.matmul(b, w.t(), out=out)) for w in W], steps, 3, reps=3)
+        t = run_graph([(lambda w=w: torch.matmul(b, w.t(), out=out)) for w in W], steps, 3, reps=3, direct_if_short=True)
         row["blas_us"] = t["us_median"]
         row["blas_note"] = ("torch.matmul (vendor BLAS) on %d rotating un-packed %s weight matrices of the same shape"
                             % (count, str(dt).replace("torch.", "")))
@@ -306,7 +332,7 @@ def main():
                 if native:
                     _lib.check(lib.mlk_re_layout_c(c.data_ptr(), c_rm.data_ptr(), m, n, st), "reLayoutC")
             return call
-        t = run_graph([mk(a) for a in A], steps, warmup)
+        t = run_graph([mk(a) for a in A], steps, warmup, direct_if_short=True)
         algo = n * k * (1 if kind == 2 else 2) + (scale.numel() * 4 if scale is not None else 0) + m * k * 2 + m * n * 2
         if native:
             algo += 2 * m * n * 2
@@ -331,7 +357,7 @@ def main():
         W = [(torch.randn((n, k), generator=gen, device=dev) * 0.02).to(dt) for _ in range(2)]
         b = torch.randn((m, k), generator=gen, device=dev).to(dt)
         out = torch.empty((m, n), dtype=dt, device=dev)
-        t = run_graph([(lambda w=w: torch.matmul(b, w.t(), out=out)) for w in W], steps, 3, reps=3)
+        t = run_graph([(lambda w=w: torch.matmul(b, w.t(), out=out)) for w in W], steps, 3, reps=3, direct_if_short=True)
         row["blas_us"] = t["us_median"]
         row["blas_tflops"] = flops / t["us_median"] / 1e6
         row["blas_note"] = "torch.matmul (vendor BLAS) on un-packed %s weights of the same shape" % str(dt).replace("torch.", "")
@@ -473,7 +499,7 @@ def main():
                     _lib.check(lib.mlk_stream_read(b.data_ptr(), nbytes, block, wgs, 0,
                                                    torch.cuda.current_stream().cuda_stream), "stream_read")
                 return call
-            t = run_graph([mk(b) for b in bufs], steps, 5, reps=3)
+            t = run_graph([mk(b) for b in bufs], steps, 5, reps=3, direct_if_short=True)
             best = max(best, nbytes / t["us_median"] / 1e3)
         return best
 
@@ -529,6 +555,7 @@ def main():
         torch.cuda.empty_cache()
         for row in per_config:
             row.pop("wall", None)
+            row.pop("how", None)
             for key in ("us", "us_median", "us_min", "gbps", "frac", "roofline_us", "ratio_to_roofline", "tflops",
                         "mfma_frac", "read_only_us", "blas_us", "blas_tflops", "traffic_over_algorithmic"):
                 if row.get(key) is not None:
@@ -552,7 +579,9 @@ def main():
         "data": "synthetic",
         "config": {"workload": head["name"], "weights": "fp16 N(0,0.02) in layout-A, %d rotating copies" % head["copies"],
                    "activations": "fp16 N(0,1) row-major [16, 4096]",
-                   "untimed_graph_replays_before_timing": settle_replays(args.steps), "launch_params": head["params"],
+                   "untimed_graph_replays_before_timing": settle_replays(args.steps),
+                   "timed_calls": head["how"],
+                   "launch_params": head["params"],
                    "algorithmic_bytes": head["bytes"]},
         "roofline": {"bound": "hbm", "achieved": round(head["gbps"], 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(head["frac"], 4), "traffic": traffic_table.get(HEAD)},

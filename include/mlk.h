@@ -170,9 +170,10 @@ int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k
  *   kernel_id 4  kernel 1 with one workgroup per CU: the N/16 row groups are dealt out as evenly as
  *                possible, two to four per workgroup (p1 and p3 are ignored).  What one CU can pull
  *                through its memory path bounds these kernels, so for few weight rows an even
- *                deal over all CUs beats a fixed p1.  16-bit weights, row-major B and C, up to 32
- *                tokens per pass, N/16 above the CU count and at most four times it; otherwise
- *                the same as kernel 1
+ *                deal over all CUs beats a fixed p1.  Up to 64 tokens, N/16 above the CU count and at
+ *                most four times it; 16-bit weights with row-major B and C from one token block on,
+ *                soft-FP8 weights or native B / C from 17 tokens on with p2 = 4 or 8 (the activations of
+ *                a k window are then shared through LDS by the waves); otherwise the same as kernel 1
  *   kernel_id 12, 14, 16, 18  kernel 1 with 2, 4, 6 or 8 k tiles in flight per wave instead of the
  *                default depth; honoured for up to 16 tokens with row-major B and C, otherwise
  *                the same as kernel 1
