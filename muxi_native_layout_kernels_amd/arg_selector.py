@@ -7,7 +7,11 @@ rows with the wrong number of cells are reported and skipped, a later row with
 the same key replaces an earlier one.  A shape that is not in its table gets a
 one-time warning and a fallback that is remembered for the rest of the process
 (arg_selector.cu:63-72, :207-224).  The tables are immutable after loading; the
-miss memo is kept under a lock.
+miss memo is kept under a lock.  Where the reference falls back to fixed
+arguments, a GEMM shape whose table holds the same weight shape at other token
+counts borrows the row of the nearest scanned count in the same kernel range
+(up to 64 tokens, or above), and only a weight shape that was never scanned
+gets arguments from a rule of thumb.
 
 What the columns select on gfx950 (the rows are produced by the scripts in
 `kernel_args_scan/`):
@@ -55,12 +59,14 @@ GEMV_FALLBACK = (256, 1, 1, 1)
 
 
 class _Selector:
-    def __init__(self, filename, key_cells, fallback, label, heuristic=None):
+    def __init__(self, filename, key_cells, fallback, label, heuristic=None, neighbours=False):
         self.filename = filename
         self.key_cells = key_cells
         self.fallback = fallback
         self.label = label
         self.heuristic = heuristic
+        self.neighbours = neighbours        # GEMM tables: a miss may borrow the row of a nearby token count
+        self._by_shape = None
         self._table = None
         self._memo = {}
         self._lock = threading.Lock()
@@ -98,6 +104,26 @@ class _Selector:
                     self._table = self._load()
         return self._table
 
+    def _neighbour(self, key):
+        """Row of the same weight shape (rows, K) at the nearest scanned token count, or None.  The tables hold a
+        few token counts per shape; the launch parameters change slowly between them, and every kernel takes any
+        token count of its range (up to 64 tokens the narrow kernels, above 64 the panel kernel), so the next
+        scanned count upwards in the same range is borrowed, else the next one downwards."""
+        if self._by_shape is None:
+            by_shape = {}
+            for (rows, tokens, k), args in self.table().items():
+                by_shape.setdefault((rows, k), []).append((tokens, args))
+            for rows_of in by_shape.values():
+                rows_of.sort()
+            self._by_shape = by_shape
+        rows, tokens, k = key
+        narrow = tokens <= 64
+        same = [(t, a) for t, a in self._by_shape.get((rows, k), ()) if (t <= 64) == narrow]
+        above = [(t, a) for t, a in same if t >= tokens]
+        if above:
+            return above[0]
+        return same[-1] if same else None
+
     def get_args(self, key):
         key = tuple(int(v) for v in key)
         hit = self.table().get(key)
@@ -107,6 +133,14 @@ class _Selector:
             memo = self._memo.get(key)
             if memo is not None:
                 return memo
+            near = self._neighbour(key) if self.neighbours else None
+            if near is not None:
+                args = near[1]
+                sys.stderr.write(" Warning: No matching arguments found for %s shape: %s. Borrowing the args of %d "
+                                 "tokens: %s\n" % (self.label, ", ".join(str(v) for v in key), near[0],
+                                                   ",".join(str(v) for v in args)))
+                self._memo[key] = args
+                return args
             args = self.heuristic(*key) if self.heuristic is not None else self.fallback
             sys.stderr.write(" Warning: No matching arguments found for %s shape: %s. Fallback args to %s\n" %
                              (self.label, ", ".join(str(v) for v in key), ",".join(str(v) for v in args)))
@@ -167,13 +201,13 @@ _SELECTORS = {
     # reference getters: csrc/arg_selector.cu:84-87 (layout gemm), :158-161 (continuous C),
     # :236-239 (gemv fp16), :312-315 (layoutA gemm), :389-392 (layoutA soft fp8), :464-467 (soft-fp8 gemv),
     # :537-540 (bf16 gemv)
-    "layout_gemm": _Selector("layout_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK, "layout GEMM", _gemm_default),
+    "layout_gemm": _Selector("layout_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK, "layout GEMM", _gemm_default, True),
     "continuous_gemm": _Selector("continuous_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK, "ContinuousC GEMM",
-                                 _gemm_default),
+                                 _gemm_default, True),
     "layoutA_gemm": _Selector("layoutA_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK, "layoutA GEMM",
-                              _gemm_default_rowmajor),
+                              _gemm_default_rowmajor, True),
     "layoutA_soft_fp8_gemm": _Selector("layoutA_Soft_Fp8_gemm_dispatch_arg.csv", 3, GEMM_FALLBACK,
-                                       "layoutA soft-FP8 GEMM", _gemm_default_rowmajor),
+                                       "layoutA soft-FP8 GEMM", _gemm_default_rowmajor, True),
     "gemv_fp16": _Selector("layout_gemv_dispatch_arg.csv", 2, GEMV_FALLBACK, "GEMV", _gemv_default),
     "gemv_bf16": _Selector("layout_gemv_bf16_dispatch_arg.csv", 2, GEMV_FALLBACK, "bf16 GEMV", _gemv_default),
     "gemv_soft_fp8": _Selector("layout_gemv_soft_fp8_dispatch_arg.csv", 2, GEMV_FALLBACK, "soft-FP8 GEMV",

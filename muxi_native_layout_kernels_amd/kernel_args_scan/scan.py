@@ -19,6 +19,7 @@ Timing: each configuration is captured `--iters` times into one HIP graph over r
 copies that together exceed the Infinity Cache, and timed with HIP events.
 """
 import argparse
+import os
 import sys
 
 import torch
@@ -50,6 +51,64 @@ DEFAULT_SHAPES = {
     "layoutA_soft_fp8_gemm": _unique(BENCH_FP8[:2] + MODEL_SHAPES),
     "continuous_gemm": _unique([(8192, 8192), (11008, 4096)] + MODEL_SHAPES),
     "layout_gemm": _unique([(8192, 8192), (11008, 4096)] + MODEL_SHAPES),
+}
+# Weight shapes (rows, K) that the reference's packaged tables hold rows for (the keys of
+# /root/reference/muxi_layout_kernels/layout_gemv_dispatch_arg.csv and layout_gemv_bf16_dispatch_arg.csv (the same
+# 90 shapes), layout_gemv_soft_fp8_dispatch_arg.csv, layoutA_gemm_dispatch_arg.csv,
+# layoutA_Soft_Fp8_gemm_dispatch_arg.csv, continuous_gemm_dispatch_arg.csv and layout_gemm_dispatch_arg.csv):
+# `--shape-set tables` scans these, so that a model served from the reference's tables finds a scanned row here too.
+_TABLE_GEMV_16BIT = [
+    (16, 4096), (16, 6144), (128, 5120), (512, 7168), (512, 8192), (896, 5120), (1024, 5120), (1024, 6144),
+    (1280, 5120), (1280, 8192), (1536, 4096), (2112, 7168), (2560, 8192), (2752, 8192), (3072, 1536), (3072,
+    8192), (3200, 5120), (3584, 3584), (3584, 18944), (4000, 6144), (4000, 8192), (4096, 1024), (4096, 4096),
+    (4096, 6144), (4096, 8192), (4096, 11008), (4096, 13696), (4608, 3584), (4608, 4096), (4608, 7168), (4992,
+    6656), (5120, 640), (5120, 1024), (5120, 3200), (5120, 3424), (5120, 3456), (5120, 5120), (5120, 8192),
+    (5120, 13824), (5120, 25600), (5504, 8192), (6144, 768), (6144, 2048), (6144, 8192), (6400, 5120), (6656,
+    1664), (6656, 4480), (6848, 5120), (6912, 5120), (7168, 256), (7168, 2048), (7168, 2304), (7168, 8192),
+    (8000, 6656), (8000, 8192), (8192, 1024), (8192, 2048), (8192, 2752), (8192, 3584), (8192, 4096), (8192,
+    5120), (8192, 5504), (8192, 7168), (8192, 7392), (8192, 14336), (8960, 6656), (10240, 5120), (11008, 4096),
+    (11008, 8192), (12288, 4096), (13696, 4096), (13824, 5120), (14336, 8192), (14784, 8192), (15360, 5120),
+    (16032, 8192), (19008, 5120), (22016, 4096), (25600, 5120), (27392, 4096), (27648, 5120), (28672, 8192),
+    (32000, 4096), (32000, 5120), (32064, 8192), (37888, 3584), (38016, 8192), (51200, 5120), (65024, 4096),
+    (125696, 4096)]
+_TABLE_GEMV_FP8 = [
+    (128, 5120), (512, 7168), (512, 8192), (1024, 5120), (1280, 5120), (2112, 7168), (3072, 1536), (3200, 5120),
+    (4096, 8192), (4608, 7168), (5120, 1024), (5120, 3200), (5120, 5120), (5120, 8192), (5120, 25600), (5120,
+    27648), (6400, 5120), (7168, 256), (7168, 2048), (7168, 2304), (7168, 5120), (8192, 4096), (8192, 5120),
+    (8192, 14336), (10240, 5120), (14336, 8192), (25600, 5120), (28672, 8192), (51200, 5120), (55296, 5120)]
+_TABLE_LAYOUTA_GEMM = [
+    (128, 5120), (512, 7168), (512, 8192), (896, 5120), (1024, 5120), (1280, 5120), (2112, 7168), (3072, 1536),
+    (3200, 5120), (4096, 8192), (4608, 7168), (5120, 640), (5120, 1024), (5120, 3200), (5120, 3456), (5120,
+    8192), (5120, 25600), (6400, 5120), (6912, 5120), (7168, 256), (7168, 2048), (7168, 2304), (8192, 4096),
+    (8192, 5120), (8192, 14336), (10240, 5120), (14336, 8192), (25600, 5120), (28672, 8192), (51200, 5120)]
+_TABLE_LAYOUTA_FP8_GEMM = [
+    (128, 5120), (512, 7168), (512, 8192), (1024, 5120), (1280, 5120), (3072, 1536), (3200, 5120), (4096, 8192),
+    (4608, 7168), (5120, 1024), (5120, 3200), (5120, 5120), (5120, 8192), (5120, 25600), (5120, 27648), (6400,
+    5120), (7168, 256), (7168, 2048), (7168, 2304), (7168, 5120), (8192, 4096), (8192, 5120), (8192, 14336),
+    (10240, 5120), (14336, 8192), (25600, 5120), (28672, 8192), (51200, 5120), (55296, 5120)]
+_TABLE_CONTINUOUS_GEMM = [
+    (128, 5120), (512, 8192), (896, 5120), (1024, 5120), (1280, 5120), (3072, 1536), (3200, 5120), (3584, 3584),
+    (3584, 18944), (4096, 8192), (4608, 3584), (4608, 7168), (5120, 640), (5120, 1024), (5120, 3200), (5120,
+    3456), (5120, 8192), (5120, 25600), (6400, 5120), (6912, 5120), (7168, 256), (7168, 2048), (7168, 2304),
+    (8192, 4096), (8192, 5120), (8192, 14336), (10240, 5120), (14336, 8192), (25600, 5120), (28672, 8192),
+    (37888, 3584), (51200, 5120)]
+_TABLE_LAYOUT_GEMM = [
+    (128, 4096), (128, 5120), (128, 6144), (512, 7168), (512, 8192), (896, 5120), (1024, 5120), (1024, 6144),
+    (1280, 5120), (1280, 8192), (1536, 4096), (2560, 8192), (2816, 8192), (3072, 1536), (3072, 8192), (3200,
+    5120), (3584, 3584), (3584, 18944), (4096, 1024), (4096, 4096), (4096, 6144), (4096, 8192), (4096, 11008),
+    (4096, 13696), (4608, 3584), (4608, 4096), (4608, 7168), (4992, 6656), (5120, 640), (5120, 1024), (5120,
+    3200), (5120, 3456), (5120, 5120), (5120, 8192), (5120, 13824), (5120, 25600), (5504, 8192), (6144, 768),
+    (6144, 8192), (6400, 5120), (6656, 1664), (6656, 4480), (6912, 5120), (7168, 256), (7168, 2048), (7168,
+    2304), (7168, 8192), (8064, 6656), (8064, 8192), (8192, 1024), (8192, 2048), (8192, 2816), (8192, 3584),
+    (8192, 4096), (8192, 5120), (8192, 5504), (8192, 7168), (8192, 7424), (8192, 14336), (8960, 6656), (10240,
+    5120), (11008, 4096), (11008, 8192), (12288, 4096), (13696, 4096), (13824, 5120), (14336, 8192), (14848,
+    8192), (15360, 5120), (16128, 8192), (19072, 5120), (22016, 4096), (25600, 5120), (27392, 4096), (27648,
+    5120), (28672, 8192), (32000, 4096), (32000, 5120), (32128, 8192), (37888, 3584), (38016, 8192), (51200,
+    5120), (65024, 4096), (125696, 4096)]
+TABLE_SHAPES = {
+    "gemv_fp16": _TABLE_GEMV_16BIT, "gemv_bf16": _TABLE_GEMV_16BIT, "gemv_soft_fp8": _TABLE_GEMV_FP8,
+    "layoutA_gemm": _TABLE_LAYOUTA_GEMM, "layoutA_soft_fp8_gemm": _TABLE_LAYOUTA_FP8_GEMM,
+    "continuous_gemm": _TABLE_CONTINUOUS_GEMM, "layout_gemm": _TABLE_LAYOUT_GEMM,
 }
 DEFAULT_TOKENS = {"layoutA_gemm": [1, 8, 16, 32, 48, 64], "layoutA_soft_fp8_gemm": [1, 4, 16, 32, 64],
                   "continuous_gemm": [16, 32, 64], "layout_gemm": [16, 32, 64]}
@@ -129,12 +188,17 @@ def scan_gemv(table, shapes, iters, progress=None):
         for block, kid, p1, p2 in grid:
             def call(a):
                 return lambda: ops.gemv_layoutA_wapper(a, x, n, k, 1, 0, block, kid, p1, p2, scale, None)
-            if not _gate(call(packed[0])(), want):
+            try:
+                if not _gate(call(packed[0])(), want):
+                    continue
+            except RuntimeError:                             # a configuration the library rejects for this shape
                 continue
             us = _time_graph([call(a) for a in packed], iters)
             if best is None or us < best[0]:
                 best = (us, block, kid, p1, p2)
         print("%s %dx%d -> %s" % (table, n, k, best), file=sys.stderr, flush=True)
+        if best is None:
+            continue
         rows.append("%d,%d,%d,%d,%d,%d" % (n, k, best[1], best[2], best[3], best[4]))
         if progress is not None:
             progress(rows[-1])
@@ -142,7 +206,7 @@ def scan_gemv(table, shapes, iters, progress=None):
     return rows
 
 
-def scan_gemm(table, shapes, tokens, iters, progress=None):
+def scan_gemm(table, shapes, tokens, iters, progress=None, known=()):
     mode, dtype = GEMM_TABLES[table]
     fp8 = mode == "fp8"
     gen = torch.Generator(device="cuda").manual_seed(2025)
@@ -152,13 +216,14 @@ def scan_gemm(table, shapes, tokens, iters, progress=None):
             print("%s %dx%d skipped: the GEMM entry points need rows and K in multiples of 128" % (table, n, k),
                   file=sys.stderr)
             continue
+        todo = [m for m in tokens if (n, m, k) not in known and not (mode in ("continuous", "native") and m % 16)]
+        if not todo:
+            continue
         plain = _weights(n, k, dtype, fp8, _copies(n * k * (1 if fp8 else 2)), gen)
         packed = [ops.pack_layout_a(w) for w in plain]
         w0 = plain[0].view(torch.float8_e4m3fn).float() if fp8 else plain[0].float()
         scale = torch.ones((n // 128, k // 128), dtype=torch.float32, device="cuda") if fp8 else None
-        for m in tokens:
-            if mode in ("continuous", "native") and m % 16:
-                continue
+        for m in todo:
             b = torch.randn((m, k), generator=gen, device="cuda").to(dtype)
             want = b.float() @ w0.t()
             b_in = ops.layoutB(b) if mode in ("continuous", "native") else b
@@ -199,7 +264,10 @@ def scan_gemm(table, shapes, tokens, iters, progress=None):
                         if mode == "continuous":
                             return lambda: ops.gemm_layoutAB_ContinuousC_wapper(a, b_in, n, m, k, 1, 0, p1, p2, p3, kid, None)
                         return lambda: ops.gemm_layoutABC_wapper(a, b_in, n, m, k, 1, 0, p1, p2, p3, kid, None)
-                    got = call(packed[0])()
+                    try:
+                        got = call(packed[0])()
+                    except RuntimeError:                     # a configuration the library rejects for this shape
+                        continue
                     if mode == "native":
                         got = ops.reLayoutC(got)
                     if not _gate(got, want):
@@ -208,6 +276,8 @@ def scan_gemm(table, shapes, tokens, iters, progress=None):
                     if best is None or us < best[0]:
                         best = (us, kid, p1, p2, p3)
             print("%s %dx%d M=%d -> %s" % (table, n, k, m, best), file=sys.stderr, flush=True)
+            if best is None:
+                continue
             rows.append("%d,%d,%d,%d,%d,%d,%d" % (n, m, k, best[1], best[2], best[3], best[4]))
             if progress is not None:
                 progress(rows[-1])
@@ -219,14 +289,19 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("table", choices=list(GEMV_TABLES) + list(GEMM_TABLES) + ["all"])
     ap.add_argument("--shapes", default=None, help="comma separated MxK weight shapes, e.g. 4096x4096,11008x4096")
+    ap.add_argument("--shape-set", choices=["default", "tables"], default="default",
+                    help="without --shapes: the benchmark and model shapes, or the shapes of the reference's tables")
+    ap.add_argument("--skip-known", action="store_true", help="leave out keys the packaged table already holds")
+    ap.add_argument("--out-dir", default=".", help="where <table>_scan_best_args.csv goes without --update")
     ap.add_argument("--tokens", default=None, help="comma separated token counts for the GEMM tables")
     ap.add_argument("--iters", type=int, default=100)
     ap.add_argument("--update", action="store_true", help="append the rows to the packaged csv")
     args = ap.parse_args()
     tables = (list(GEMV_TABLES) + list(GEMM_TABLES)) if args.table == "all" else [args.table]
     for table in tables:
-        shapes = DEFAULT_SHAPES[table] if args.shapes is None else \
+        shapes = (TABLE_SHAPES if args.shape_set == "tables" else DEFAULT_SHAPES)[table] if args.shapes is None else \
             [tuple(int(v) for v in s.split("x")) for s in args.shapes.split(",")]
+        known = set(arg_selector.selector(table).table()) if args.skip_known else set()
         gemv = table in GEMV_TABLES
         header = "m,k,BLOCK_DIM_X,KernelId,KernelParam1,KernelParam2" if gemv else \
             "m,n,k,kernelId,kernelParam1,kernelParam2,kernelParam3"
@@ -234,7 +309,7 @@ def main():
             path = arg_selector.selector(table).path()
             out = open(path, "a")
         else:
-            path = "%s_scan_best_args.csv" % table
+            path = os.path.join(args.out_dir, "%s_scan_best_args.csv" % table)
             out = open(path, "w")
             out.write(header + "\n")
 
@@ -242,10 +317,10 @@ def main():
             out.write(row + "\n")
             out.flush()
         if gemv:
-            rows = scan_gemv(table, shapes, args.iters, progress)
+            rows = scan_gemv(table, [s for s in shapes if s not in known], args.iters, progress)
         else:
             tokens = DEFAULT_TOKENS[table] if args.tokens is None else [int(v) for v in args.tokens.split(",")]
-            rows = scan_gemm(table, shapes, tokens, args.iters, progress)
+            rows = scan_gemm(table, shapes, tokens, args.iters, progress, known)
         out.close()
         print("wrote %d rows to %s" % (len(rows), path), file=sys.stderr)
 

@@ -89,6 +89,37 @@ def test_product_selector_reads_table(tmp_path):
     assert sel.get_args((128, 16, 256)) == (1, 4, 8, 1)
 
 
+def test_gemm_miss_borrows_the_nearest_scanned_token_count(capsys, tmp_path):
+    """A GEMM key whose weight shape is in the table at other token counts takes the next scanned count upwards in
+    the same kernel range (up to 64 tokens / above), else the next one downwards; an unknown weight shape takes the
+    rule of thumb.  GeMV selectors never borrow."""
+    p = tmp_path / "t.csv"
+    p.write_text("m,n,k,kernelId,kernelParam1,kernelParam2,kernelParam3\n"
+                 "4096,8,4096,14,1,4,1\n4096,32,4096,4,1,8,1\n4096,64,4096,2,2,1,1\n"
+                 "4096,256,4096,3,4,1,2\n4096,1024,4096,3,4,2,1\n8192,16,1024,1,2,2,1\n")
+    sel = arg_selector._Selector(str(p), 3, arg_selector.GEMM_FALLBACK, "tmp", lambda n, m, k: (9, 9, 9, 9), True)
+    sel.path = lambda: str(p)
+    assert sel.get_args((4096, 32, 4096)) == (4, 1, 8, 1)        # a hit stays a hit
+    assert sel.get_args((4096, 1, 4096)) == (14, 1, 4, 1)        # up to the 8-token row
+    assert sel.get_args((4096, 24, 4096)) == (4, 1, 8, 1)
+    assert sel.get_args((4096, 33, 4096)) == (2, 2, 1, 1)
+    assert sel.get_args((4096, 100, 4096)) == (3, 4, 1, 2)       # above 64 tokens only the rows above 64 count
+    assert sel.get_args((4096, 512, 4096)) == (3, 4, 2, 1)
+    assert sel.get_args((4096, 4096, 4096)) == (3, 4, 2, 1)      # nothing above: the largest scanned count
+    assert sel.get_args((8192, 48, 1024)) == (1, 2, 2, 1)        # nothing above in the range: downwards
+    assert sel.get_args((8192, 128, 1024)) == (9, 9, 9, 9)       # no row above 64 tokens for this shape
+    assert sel.get_args((1024, 16, 1024)) == (9, 9, 9, 9)        # weight shape never scanned
+    err = capsys.readouterr().err
+    assert err.count("Borrowing the args of") == 7 and err.count("Fallback args to") == 2
+    plain = arg_selector._Selector(str(p), 3, arg_selector.GEMM_FALLBACK, "tmp")
+    plain.path = lambda: str(p)
+    assert plain.get_args((4096, 24, 4096)) == (1, 1, 1, 1)
+    for name in ("gemv_fp16", "gemv_bf16", "gemv_soft_fp8"):
+        assert not arg_selector.selector(name).neighbours
+    for name in ("layout_gemm", "continuous_gemm", "layoutA_gemm", "layoutA_soft_fp8_gemm"):
+        assert arg_selector.selector(name).neighbours
+
+
 def test_gemv_guard_product():
     assert arg_selector.gemv_guard((512, 1, 2, 4), 4096, 4096) == (512, 1, 2, 4)
     assert arg_selector.gemv_guard((512, 1, 3, 4), 4096, 4096) == (256, 1, 1, 4)
