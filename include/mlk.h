@@ -174,6 +174,12 @@ int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k
  *                most four times it; 16-bit weights with row-major B and C from one token block on,
  *                soft-FP8 weights or native B / C from 17 tokens on with p2 = 4 or 8 (the activations of
  *                a k window are then shared through LDS by the waves); otherwise the same as kernel 1
+ *   kernel_id 5  kernel 3 with the K slices (p3) applied only to the panels that are left over after whole
+ *                rounds of one panel per CU: with one workgroup per CU the grid runs in rounds, and a last
+ *                round that fills a third of the chip costs as much as a full one; slicing just its panels
+ *                p3 ways puts the idle CUs to work without paying the fold on every panel.  The same as
+ *                kernel 3 when there is no whole round, and kernel 3 with p3 = 1 when nothing is left over or
+ *                when the token tiles of a row tile do not divide an XCD's CUs.  Workspace as for kernel 3
  *   kernel_id 12, 14, 16, 18  kernel 1 with 2, 4, 6 or 8 k tiles in flight per wave instead of the
  *                default depth; honoured for up to 16 tokens with row-major B and C, otherwise
  *                the same as kernel 1

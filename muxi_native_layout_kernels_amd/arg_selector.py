@@ -41,6 +41,8 @@ What the columns select on gfx950 (the rows are produced by the scripts in
                                  and from 17 tokens on with kernelParam2 = 8, the activations of a k
                                  window are shared through LDS by up to eight waves; kernelParam1
                                  and kernelParam3 are not used; otherwise the same as 1)
+                             5 = kernel 3 with the K slices (kernelParam3) applied only to the panels left
+                                 over after whole rounds of one panel per CU
                              12, 14, 16, 18 = kernel 1 with 2, 4, 6, 8 k tiles in flight per
                                  wave (up to 16 tokens, row-major activations and output;
                                  otherwise the same as 1)

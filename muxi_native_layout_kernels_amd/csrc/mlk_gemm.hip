@@ -57,8 +57,8 @@ extern template int launch_modes<BF16, true>(const GemmArgs &, int, int, int, in
 // kernel id 3 (mlk_panel.hip)
 size_t panel_partial_bytes(int m, int n, int sk);
 int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int a_kind, float alpha, const void *bias,
-                 const float *scale, int width, int rows, int sk, void *counters, size_t counter_bytes, void *partial,
-                 size_t partial_bytes, hipStream_t s);
+                 const float *scale, int width, int rows, int sk, bool last_round_only, void *counters,
+                 size_t counter_bytes, void *partial, size_t partial_bytes, hipStream_t s);
 
 }  // namespace mlk
 
@@ -87,11 +87,11 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
     MLK_REQUIRE(m >= 0 && n >= 0 && k >= 0, "gemm: negative size");
     MLK_REQUIRE(n % 16 == 0, "gemm: N % 16 must be 0");
     MLK_REQUIRE(k % 32 == 0, "gemm: K % 32 must be 0");
-    MLK_REQUIRE(kernel_id == 1 || kernel_id == 2 || kernel_id == 3 || kernel_id == 4 || kernel_id == 12 || kernel_id == 14 || kernel_id == 16 ||
+    MLK_REQUIRE(kernel_id == 1 || kernel_id == 2 || kernel_id == 3 || kernel_id == 4 || kernel_id == 5 || kernel_id == 12 || kernel_id == 14 || kernel_id == 16 ||
                     kernel_id == 18,
                 "gemm: unknown kernel id");
     MLK_REQUIRE(p1 == 1 || p1 == 2 || p1 == 4 || p1 == 8, "gemm: row groups per wave (p1) must be 1, 2, 4 or 8");
-    MLK_REQUIRE(kernel_id == 3 || (n / 16) % p1 == 0, "gemm: row groups per wave (p1) must divide N/16");
+    MLK_REQUIRE(kernel_id == 3 || kernel_id == 5 || (n / 16) % p1 == 0, "gemm: row groups per wave (p1) must divide N/16");
     MLK_REQUIRE(p2 == 1 || p2 == 2 || p2 == 4 || p2 == 8 || p2 == 16, "gemm: waves per workgroup (p2) must be 1, 2, 4, 8 or 16");
     MLK_REQUIRE(p3 >= 1 && p3 <= 64, "gemm: K splits across workgroups (p3) must be 1..64");
     MLK_REQUIRE(x_kind == MLK_F16 || x_kind == MLK_BF16, "gemm: activations must be fp16 or bf16");
@@ -109,8 +109,9 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
     }
     if (m == 0 || n == 0) return MLK_OK;
     MLK_REQUIRE(a && b && c, "gemm: null pointer");
-    if (kernel_id == 3) {
-        // panel kernel: any number of tokens in one launch; p1 = row groups per wave (2: 128-row panels, 4: 256-row
+    if (kernel_id == 3 || kernel_id == 5) {
+        // panel kernel: any number of tokens in one launch; kernel id 5 slices only the panels of the last, partial
+        // round of one panel per CU; p1 = row groups per wave (2: 128-row panels, 4: 256-row
         // panels, else chosen from the shape); p2 = tokens per panel (1: 128, 2: 256, else chosen from the shape);
         // p3 = K slices (one slice up to 64 tokens, where the
         // workspace is sized for the narrow kernels)
@@ -119,7 +120,7 @@ extern "C" int mlk_gemm_layout_a(const void *a, const void *b, void *c, int m, i
         uint8_t *ws = (uint8_t *)workspace;
         const size_t part_bytes = workspace_bytes > kCounterBytes ? workspace_bytes - kCounterBytes : 0;
         return launch_panel(a, b, c, m, n, k, fp8 ? MLK_FP8_E4M3 : x_kind, alpha, bias, scale, p2 == 1 ? 128 : (p2 == 2 ? 256 : 0),
-                            p1 == 2 ? 128 : (p1 == 4 ? 256 : 0), m > 64 ? p3 : 1, ws, kCounterBytes,
+                            p1 == 2 ? 128 : (p1 == 4 ? 256 : 0), m > 64 ? p3 : 1, kernel_id == 5, ws, kCounterBytes,
                             ws ? ws + kCounterBytes : nullptr, ws ? part_bytes : 0, (hipStream_t)stream);
     }
     int sk = p3;

@@ -37,10 +37,11 @@ struct PanelArgs {
     uint16_t *C;
     const uint16_t *bias;
     const float *scale;
-    f32x4 *partial;      // [SK][tiles][4 waves][quads of a wave][two planes of 64 x 8 bytes]
-    int *counters;       // [tiles], zero between calls
+    f32x4 *partial;      // [SK][sliced tiles][4 waves][quads of a wave][two planes of 64 x 8 bytes]
+    int *counters;       // [sliced tiles], zero between calls
     int M, N, K;
-    int SK;
+    int SK;              // K slices of the row tiles from whole_groups * 8 on
+    int whole_groups;    // groups of eight row tiles in front that are not sliced (0: every row tile has SK slices)
     int row_tiles, token_tiles;
     float alpha;
 };
@@ -54,21 +55,26 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
 
-    // workgroup -> (row tile, k slice, token tile)
+    // workgroup -> (row tile, k slice, token tile): per XCD first the groups of eight row tiles that are computed
+    // whole, then the sliced ones
     const int xcd = blockIdx.x & 7;
     int u = blockIdx.x >> 3;
+    const int whole_wgs = p.whole_groups * p.token_tiles;
+    const bool sliced = u >= whole_wgs;
+    const int SK = sliced ? p.SK : 1;
+    if (sliced) u -= whole_wgs;
     const int tt = u % p.token_tiles;
     u /= p.token_tiles;
-    const int sk = u % p.SK;
-    const int rt = (u / p.SK) * 8 + xcd;
+    const int sk = u % SK;
+    const int rt = ((sliced ? p.whole_groups : 0) + u / SK) * 8 + xcd;
     if (rt >= p.row_tiles) return;                            // the grid is padded to whole groups of eight row tiles
 
     const int groups = p.N >> 4;
     const int rg0 = (rt * kTileWaves + wave) * R;
     const int tok0 = tt * (TB * 32);
     const int nwin_total = p.K / (KW * 32);
-    const int wbeg = (int)((long long)sk * nwin_total / p.SK);
-    const int nwin = (int)((long long)(sk + 1) * nwin_total / p.SK) - wbeg;
+    const int wbeg = (int)((long long)sk * nwin_total / SK);
+    const int nwin = (int)((long long)(sk + 1) * nwin_total / SK) - wbeg;
     const int scale_cols = (p.K + 127) >> 7;
 
     const uint8_t *abase[R];                                  // wave-uniform; the lane offset is added per load
@@ -118,7 +124,7 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
         store4<T>(p.C + (size_t)tok * p.N + n, o[0], o[1], o[2], o[3]);
     };
     auto quad = [&](const f32x16 &v, int g) { return f32x4{v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3]}; };
-    if (p.SK == 1) {
+    if (SK == 1) {
 #pragma unroll
         for (int pr = 0; pr < PR; ++pr)
 #pragma unroll
@@ -127,8 +133,8 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
                 for (int g = 0; g < 4; ++g) epilogue(pr, tb, g, quad(acc[pr][tb], g));
         return;
     }
-    const int tile = rt * p.token_tiles + tt;
-    const int tiles = p.row_tiles * p.token_tiles;
+    const int tile = (rt - p.whole_groups * 8) * p.token_tiles + tt;               // among the sliced tiles
+    const int tiles = (p.row_tiles - p.whole_groups * 8) * p.token_tiles;
     // 64-lane group of quad jj of this wave in slice s (two planes of 8-byte halves, see st_agent_planar)
     auto group_at = [&](int s, int jj) -> f32x4 * {
         return p.partial + ((((size_t)s * tiles + tile) * kTileWaves + wave) * (PR * TB * 4) + jj) * 64;
@@ -145,7 +151,7 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     __syncthreads();
     if (threadIdx.x == 0) {
         int prev = __hip_atomic_fetch_add(&p.counters[tile], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (prev == p.SK - 1);
+        s_last = (prev == SK - 1);
         if (s_last) __hip_atomic_store(&p.counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
     __syncthreads();
@@ -170,11 +176,11 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
                 for (int e = 0; e < 16; ++e) acc[pr][tb][e] += t[tb * 4 + (e >> 2)][e & 3];
         };
         fetch(t0, 0);
-        for (int sl = 0; sl < p.SK; sl += 2) {
-            if (sl + 1 < p.SK) fetch(t1, sl + 1);
+        for (int sl = 0; sl < SK; sl += 2) {
+            if (sl + 1 < SK) fetch(t1, sl + 1);
             add(t0);
-            if (sl + 1 < p.SK) {
-                if (sl + 2 < p.SK) fetch(t0, sl + 2);
+            if (sl + 1 < SK) {
+                if (sl + 2 < SK) fetch(t0, sl + 2);
                 add(t1);
             }
         }
@@ -205,10 +211,11 @@ size_t panel_partial_bytes(int m, int n, int sk) {
 
 // a_kind: MLK_F16, MLK_BF16 or MLK_FP8_E4M3 (bf16 activations); width: tokens per panel (128 or 256), anything else =
 // panel_tokens(m, n); rows: weight rows per panel (128 or 256; 128 only with 128 tokens), anything else = chosen
-// from the number of panels
+// from the number of panels; sk: K slices; last_round_only: slice only the panels that are left over after whole
+// rounds of one panel per CU (every panel when there is no whole round, none when nothing is left over)
 int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int a_kind, float alpha, const void *bias,
-                 const float *scale, int width, int rows, int sk, void *counters, size_t counter_bytes, void *partial,
-                 size_t partial_bytes, hipStream_t s) {
+                 const float *scale, int width, int rows, int sk, bool last_round_only, void *counters,
+                 size_t counter_bytes, void *partial, size_t partial_bytes, hipStream_t s) {
     PanelArgs p;
     p.A = (const uint8_t *)a;
     p.B = (const uint16_t *)b;
@@ -240,13 +247,24 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
         rows = panels256 * 8 <= (long long)cus * 3 ? 128 : 256;
     }
     p.row_tiles = (n + rows - 1) / rows;
+    const int groups = (p.row_tiles + 7) / 8;                 // groups of eight row tiles, one per XCD
+    p.whole_groups = 0;
+    if (last_round_only && sk > 1) {
+        // workgroups start in the order of their ids, eight XCDs taking turns: a round is CUs / 8 workgroups per XCD
+        const int per_xcd = device_cus() / 8;
+        if (p.token_tiles <= per_xcd && per_xcd % p.token_tiles == 0) {
+            const int groups_per_round = per_xcd / p.token_tiles;
+            p.whole_groups = groups / groups_per_round * groups_per_round;
+        }
+        if (p.whole_groups == groups) p.whole_groups = 0, p.SK = sk = 1;    // nothing left over
+    }
     if (sk > 1) {
         MLK_REQUIRE(partial != nullptr && counters != nullptr, "gemm: a K split across workgroups needs a workspace");
         MLK_REQUIRE((size_t)p.row_tiles * p.token_tiles * sizeof(int) <= counter_bytes,
                     "gemm: too many panels for the counter region");
         if (partial_bytes < panel_partial_bytes(m, n, sk)) return fail(MLK_ERR_WORKSPACE, "gemm: workspace too small");
     }
-    const int grid = ((p.row_tiles + 7) / 8) * 8 * p.token_tiles * sk;
+    const int grid = (p.whole_groups + (groups - p.whole_groups) * sk) * 8 * p.token_tiles;
     // one workgroup per CU (the register ring and the accumulators take a whole SIMD's file); more than 64 KiB of
     // dynamic LDS has to be requested once per kernel
 #define MLK_PANEL(TT, F8, TBB, PRR)                                                                                    \

@@ -206,7 +206,7 @@ def scan_gemv(table, shapes, iters, progress=None):
     return rows
 
 
-def scan_gemm(table, shapes, tokens, iters, progress=None, known=()):
+def scan_gemm(table, shapes, tokens, iters, progress=None, known=(), kernel_ids=None):
     mode, dtype = GEMM_TABLES[table]
     fp8 = mode == "fp8"
     gen = torch.Generator(device="cuda").manual_seed(2025)
@@ -251,8 +251,10 @@ def scan_gemm(table, shapes, tokens, iters, progress=None, known=()):
             if mode in ("rowmajor", "fp8") and m > 64 and k % 128 == 0:
                 grid = [g for g in grid if g[0] != 1]
                 grid += [(3, rg, w, sk) for rg, w in ((2, 1), (4, 1), (4, 2)) for sk in (1, 2, 4) if (k // 128) // sk >= 2]
+                # kernel 5: the same with only the panels of the last, partial round sliced
+                grid += [(5, rg, w, sk) for rg, w in ((2, 1), (4, 1), (4, 2)) for sk in (2, 3, 4) if (k // 128) // sk >= 2]
             for kid, p1, p2, p3 in grid:
-                if (n // 16) % p1:
+                if (n // 16) % p1 or (kernel_ids is not None and kid not in kernel_ids):
                     continue
                 if True:
                     def call(a):
@@ -293,6 +295,7 @@ def main():
                     help="without --shapes: the benchmark and model shapes, or the shapes of the reference's tables")
     ap.add_argument("--skip-known", action="store_true", help="leave out keys the packaged table already holds")
     ap.add_argument("--out-dir", default=".", help="where <table>_scan_best_args.csv goes without --update")
+    ap.add_argument("--kernel-ids", default=None, help="GEMM tables: only these kernel ids, e.g. 3,5")
     ap.add_argument("--tokens", default=None, help="comma separated token counts for the GEMM tables")
     ap.add_argument("--iters", type=int, default=100)
     ap.add_argument("--update", action="store_true", help="append the rows to the packaged csv")
@@ -320,7 +323,8 @@ def main():
             rows = scan_gemv(table, [s for s in shapes if s not in known], args.iters, progress)
         else:
             tokens = DEFAULT_TOKENS[table] if args.tokens is None else [int(v) for v in args.tokens.split(",")]
-            rows = scan_gemm(table, shapes, tokens, args.iters, progress, known)
+            ids = None if args.kernel_ids is None else {int(v) for v in args.kernel_ids.split(",")}
+            rows = scan_gemm(table, shapes, tokens, args.iters, progress, known, ids)
         out.close()
         print("wrote %d rows to %s" % (len(rows), path), file=sys.stderr)
 

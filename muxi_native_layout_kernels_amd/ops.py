@@ -270,7 +270,8 @@ def _gemm_call(A, A_Scale, B, m, n, k, alpha, beta, bias, b_mode, c_mode, kernel
 
 def _gemm_guard(args, m):
     kid, p1, p2, p3 = args
-    if kid not in (1, 2, 3, 4, 12, 14, 16, 18) or p1 not in (1, 2, 4, 8) or (kid != 3 and (m // 16) % p1 != 0) or \
+    if kid not in (1, 2, 3, 4, 5, 12, 14, 16, 18) or p1 not in (1, 2, 4, 8) or \
+            (kid not in (3, 5) and (m // 16) % p1 != 0) or \
             p2 not in (1, 2, 4, 8, 16) or p3 < 1:
         return (1, 1, 4, 1)
     return args

@@ -183,6 +183,43 @@ def test_gemm_panel_kernel_soft_fp8(mlk, m, scaled):
         assert_close(c, want, RTOL, ATOL, "panel fp8 M=%d slices=%d width=%d" % (m, p3, width))
 
 
+@pytest.mark.parametrize("n,m,k,p1,p2,p3", [
+    (5504, 1024, 256, 2, 1, 2),      # 43 row tiles x 8 token tiles of 128 x 128: one whole round of 256 panels + 88 sliced
+    (5520, 1000, 512, 2, 1, 3),      # ragged rows and tokens, three uneven slices of four windows
+    (16640, 1024, 256, 4, 2, 2),     # 65 row tiles x 4 token tiles of 256 x 256: 256 whole + 4 sliced
+    (11008, 1024, 128, 4, 1, 2),     # one window: a single slice does all the work
+    (5504, 384, 256, 2, 1, 2),       # three token tiles do not divide an XCD's CUs: every panel whole
+    (2048, 1024, 256, 2, 1, 2),      # exactly one round: nothing left over, no slices
+    (1024, 200, 512, 4, 1, 4),       # less than a round: every panel sliced, as with kernelId 3
+])
+def test_gemm_panel_kernel_last_round_slices(mlk, n, m, k, p1, p2, p3):
+    """kernelId 5: the panel kernel with K slices only on the panels left over after whole rounds of one panel per
+    CU; bit-equal on a second run, and equal to the oracle like kernelId 3."""
+    dtype = torch.bfloat16
+    w = randn((n, k), dtype, 0.05, 191)
+    b = randn((m, k), dtype, 1.0, 192)
+    bias = randn((1, n), dtype, 1.0, 193)
+    a = pack_a(w).cuda()
+    c = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=p1, kernelParam2=p2, kernelParam3=p3,
+                                kernelId=5, bias=bias.cuda())
+    assert c.shape == (m, n) and c.dtype == dtype
+    assert_close(c, ogemm.linear_expected(w, b, 0.5, bias), RTOL, ATOL, "panel, last round sliced n=%d M=%d" % (n, m))
+    c2 = mlk.gemm_layoutA_wapper(a, b.cuda(), n, m, k, alpha=0.5, kernelParam1=p1, kernelParam2=p2, kernelParam3=p3,
+                                 kernelId=5, bias=bias.cuda())
+    assert torch.equal(c, c2)
+
+
+def test_gemm_panel_kernel_last_round_slices_soft_fp8(mlk):
+    n, k, m = 5504, 512, 1024
+    codes = fp8_codes((n, k), 195)
+    g = torch.Generator().manual_seed(196)
+    scale = (torch.rand((n // 128, k // 128), generator=g) * 0.02 + 0.001).float()
+    b = randn((m, k), torch.bfloat16, 1.0, 197)
+    c = mlk.gemm_layoutA_soft_fp8_wapper(pack_a(codes).cuda(), scale.cuda(), b.cuda(), n, m, k, kernelParam1=2,
+                                         kernelParam2=1, kernelParam3=2, kernelId=5)
+    assert_close(c, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), b), RTOL, ATOL, "panel fp8, last round sliced")
+
+
 def test_gemm_panel_kernel_is_the_wide_default(mlk):
     """Above 64 tokens the heuristic for unscanned shapes picks the panel kernel; a K that is no
     multiple of 128 keeps the row-shared kernel, and the panel kernel refuses it when asked for by id."""

@@ -16,7 +16,9 @@ def test_gemm_guard_accepts_both_kernels_and_rejects_bad_rows():
     assert ops._gemm_guard((18, 8, 4, 1), 28672) == (18, 8, 4, 1)    # eight row groups per wave
     assert ops._gemm_guard((3, 1, 1, 2), 11008) == (3, 1, 1, 2)      # panel kernel
     assert ops._gemm_guard((3, 2, 4, 2), 272) == (3, 2, 4, 2)        # its row groups per wave need not divide N/16
-    assert ops._gemm_guard((5, 1, 1, 1), 11008) == (1, 1, 4, 1)      # unknown kernel id
+    assert ops._gemm_guard((5, 4, 1, 2), 11008) == (5, 4, 1, 2)      # panel kernel, last round sliced
+    assert ops._gemm_guard((5, 2, 4, 3), 272) == (5, 2, 4, 3)
+    assert ops._gemm_guard((6, 1, 1, 1), 11008) == (1, 1, 4, 1)      # unknown kernel id
     assert ops._gemm_guard((1, 3, 4, 1), 11008) == (1, 1, 4, 1)      # row groups per wave not in {1,2,4}
     assert ops._gemm_guard((1, 4, 4, 1), 16 * 6) == (1, 1, 4, 1)     # 6 row groups are not a multiple of 4
     assert ops._gemm_guard((1, 1, 5, 1), 4096) == (1, 1, 4, 1)       # waves per workgroup not a power of two
