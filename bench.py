@@ -115,6 +115,12 @@ def main():
                 out.append((torch.randn((n // 16, k // 8, 16, 8), generator=gen, device=dev) * 0.02).to(DT[kind]))
         return out
 
+    def block_scales(shape):
+        """fp32 block scales of soft-FP8 weights: arbitrary values, as in the reference's scripts (a scale matrix drawn
+        at random, benchmark_and_test/gemv_benchmark_soft_fp8.py:30), so the kernels take their general widening
+        path; scales that are all exact powers of two take a cheaper one and are timed on one extra line."""
+        return torch.rand(shape, generator=gen, device=dev) * 0.02 + 0.001
+
     bench_stream = torch.cuda.Stream()      # every timed region runs on this one stream
 
     def settle_replays(steps):
@@ -265,13 +271,16 @@ def main():
                            "logical CPUs" % (slab, I, T, reps, dt_s * 1e3, host_cpus))
 
     # ------------------------------------------------------------------ GPU cases
-    def gemv_case(name, n, k, kind, steps, warmup, yardstick=False, cpu_rows=2048):
+    def gemv_case(name, n, k, kind, steps, warmup, yardstick=False, cpu_rows=2048, unit_scales=False):
         xk = 1 if kind == 2 else kind
         wbytes = n * k * (1 if kind == 2 else 2)
         A = weights(n, k, kind, copies_for(wbytes))
         x = torch.randn((1, k), generator=gen, device=dev).to(DT[xk])
         y = torch.empty((1, n), dtype=DT[xk], device=dev)
-        scale = torch.ones(((n + 127) // 128, (k + 127) // 128), dtype=torch.float32, device=dev) if kind == 2 else None
+        scale = None
+        if kind == 2:
+            scale = torch.ones(((n + 127) // 128, (k + 127) // 128), dtype=torch.float32, device=dev) if unit_scales \
+                else block_scales(((n + 127) // 128, (k + 127) // 128))
         sel = {0: "gemv_fp16", 1: "gemv_bf16", 2: "gemv_soft_fp8"}[kind]
         block, kid, p1, p2 = arg_selector.gemv_guard(arg_selector.selector(sel).get_args((n, k)), n, k)
 
@@ -288,7 +297,8 @@ def main():
         del A
         if yardstick:
             extra["read_only_us"] = read_only_us(wbytes, steps)
-        extra["cpu_baseline"] = cpu_linear(n, k, 1, kind, cpu_rows)
+        if cpu_rows:
+            extra["cpu_baseline"] = cpu_linear(n, k, 1, kind, cpu_rows)
         return finish(name, t, algo, **extra)
 
     def blas_yardstick(row, n, k, dt, m, steps, count):
@@ -306,7 +316,7 @@ def main():
         xk = 1 if kind == 2 else kind
         A = weights(n, k, kind, copies or copies_for(n * k * (1 if kind == 2 else 2)))
         b = torch.randn((m, k), generator=gen, device=dev).to(DT[xk])
-        scale = torch.ones((n // 128, k // 128), dtype=torch.float32, device=dev) if kind == 2 else None
+        scale = block_scales((n // 128, k // 128)) if kind == 2 else None
         table = "layoutA_soft_fp8_gemm" if kind == 2 else ("layout_gemm" if native else "layoutA_gemm")
         kid, p1, p2, p3 = mlk.ops._gemm_guard(arg_selector.selector(table).get_args((n, m, k)), n)
         if native:
@@ -376,8 +386,8 @@ def main():
                 w1 = w1.to(torch.float8_e4m3fn).view(torch.uint8)
                 w2 = (torch.randn((E, H, I), generator=gen, device=dev) * 16).clamp_(-448, 448)
                 w2 = w2.to(torch.float8_e4m3fn).view(torch.uint8)
-                s1 = torch.ones((E, 2 * I // 128, H // 128), dtype=torch.float32, device=dev)
-                s2 = torch.ones((E, H // 128, I // 128), dtype=torch.float32, device=dev)
+                s1 = block_scales((E, 2 * I // 128, H // 128))
+                s2 = block_scales((E, H // 128, I // 128))
                 moe_w[key] = (w1, w2, s1, s2)
             else:
                 w1 = (torch.randn((E, 2 * I, H), generator=gen, device=dev) * 0.02).to(torch.bfloat16)
@@ -531,6 +541,8 @@ def main():
             add(gemm_case, "C2 fp16 gemm_layoutA 11008x4096 M=%d" % m, N, K_, 0, m, short, 10, blas=True)
         add(gemv_case, "C2 fp16 gemv 11008x4096", N, K_, 0, short, 10)
         add(gemv_case, "C3 soft-fp8 gemv 28672x8192", 28672, 8192, 2, short, 10, yardstick=True, cpu_rows=1024)
+        add(gemv_case, "C3 soft-fp8 gemv 28672x8192, power-of-two block scales", 28672, 8192, 2, short, 10, cpu_rows=0,
+            unit_scales=True)
         for m in (4, 16):
             add(gemm_case, "C3 soft-fp8 gemm_layoutA 28672x8192 M=%d" % m, 28672, 8192, 2, m, short, 10, cpu_rows=1024)
         add(gemm_case, "C4 bf16 gemm_layoutABC+reLayoutC 8192x8192 M=32", 8192, 8192, 1, 32, short, 10, native=True,

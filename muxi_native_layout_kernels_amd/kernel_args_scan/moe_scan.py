@@ -94,8 +94,9 @@ def scan(experts, topk, hidden, inter, grouped, fp8, tokens, iters, out):
         w1 = w1.to(torch.float8_e4m3fn).view(torch.uint8)
         w2 = (torch.randn((experts, hidden, inter), generator=gen, device=dev) * 16).clamp_(-448, 448)
         w2 = w2.to(torch.float8_e4m3fn).view(torch.uint8)
-        kw = dict(w1_scale=torch.full((experts, 2 * inter // 128, hidden // 128), 2.0 ** -10, device=dev),
-                  w2_scale=torch.full((experts, hidden // 128, inter // 128), 2.0 ** -10, device=dev),
+        # arbitrary block scales: the general widening path (powers of two would take a cheaper one)
+        kw = dict(w1_scale=torch.rand((experts, 2 * inter // 128, hidden // 128), generator=gen, device=dev) * 2e-3 + 1e-4,
+                  w2_scale=torch.rand((experts, hidden // 128, inter // 128), generator=gen, device=dev) * 2e-3 + 1e-4,
                   block_shape=[128, 128], soft_fp8=True)
     else:
         w1 = (torch.randn((experts, 2 * inter, hidden), generator=gen, device=dev) * 0.02).to(dtype)

@@ -156,6 +156,21 @@ def _weights(n, k, dtype, fp8, count, gen):
     return out
 
 
+def _block_scales(rows, cols, gen):
+    """fp32 block scales of soft-FP8 weights with arbitrary values (the general widening path; scales that are all
+    powers of two would take a cheaper one and tune the tables for a special case)."""
+    return torch.rand((rows, cols), generator=gen, device="cuda") * 0.02 + 0.001
+
+
+def _scaled(codes, scale):
+    """Value of soft-FP8 weights as the kernels widen them: e4m3 code times the fp32 scale of its 128 x 128 block,
+    low 16 bits dropped (a bf16 by truncation)."""
+    n, k = codes.shape
+    full = scale.repeat_interleave(128, 0)[:n].repeat_interleave(128, 1)[:, :k]
+    wide = codes.view(torch.float8_e4m3fn).float() * full
+    return (wide.view(torch.int32) & -65536).view(torch.float32)
+
+
 def _copies(nbytes):
     return int(max(2, min(16, (3 * MALL_BYTES + nbytes - 1) // nbytes)))
 
@@ -175,8 +190,8 @@ def scan_gemv(table, shapes, iters, progress=None):
         plain = _weights(n, k, xdt, fp8, _copies(n * k * (1 if fp8 else 2)), gen)
         packed = [ops.pack_layout_a(w) for w in plain]
         x = torch.randn((1, k), generator=gen, device="cuda").to(xdt)
-        scale = torch.ones(((n + 127) // 128, (k + 127) // 128), dtype=torch.float32, device="cuda") if fp8 else None
-        w0 = plain[0].view(torch.float8_e4m3fn).float() if fp8 else plain[0].float()
+        scale = _block_scales((n + 127) // 128, (k + 127) // 128, gen) if fp8 else None
+        w0 = _scaled(plain[0], scale) if fp8 else plain[0].float()
         want = x.float() @ w0.t()
         best = None
         # kernel 1: (threads, row groups per workgroup, loads in flight); kernels 2 and 3 (soft-FP8 only):
@@ -221,8 +236,8 @@ def scan_gemm(table, shapes, tokens, iters, progress=None, known=(), kernel_ids=
             continue
         plain = _weights(n, k, dtype, fp8, _copies(n * k * (1 if fp8 else 2)), gen)
         packed = [ops.pack_layout_a(w) for w in plain]
-        w0 = plain[0].view(torch.float8_e4m3fn).float() if fp8 else plain[0].float()
-        scale = torch.ones((n // 128, k // 128), dtype=torch.float32, device="cuda") if fp8 else None
+        scale = _block_scales(n // 128, k // 128, gen) if fp8 else None
+        w0 = _scaled(plain[0], scale) if fp8 else plain[0].float()
         for m in todo:
             b = torch.randn((m, k), generator=gen, device="cuda").to(dtype)
             want = b.float() @ w0.t()
