@@ -426,7 +426,8 @@ def test_fused_moe_mixtral_shape(mlk, T):
 @pytest.mark.parametrize("T,unit_scales", [(1, False), (16, True), (16, False), (64, False), (256, False)])
 def test_fused_moe_mixtral_shape_soft_fp8(mlk, T, unit_scales):
     """The soft-FP8 variant of the same layer: e4m3 bytes from N(0, 1) * 16 clipped to +-448, one fp32 scale per
-    128 x 128 block (all ones as the benchmark runs it, or random factors around 1e-3)."""
+    128 x 128 block (random factors around 1e-3, the general widening path; or all ones, which are powers of two and
+    take the scaled converter)."""
     from muxi_native_layout_kernels_amd.moe_planC import fused_moe
     from oracle import softfp8
     E, K, H, I = 8, 2, 4096, 14336
