@@ -171,7 +171,8 @@ int mlk_gemv_layout_a(const void *a, const void *x, void *y, int m, int n, int k
  *                possible, two to four per workgroup (p1 and p3 are ignored).  What one CU can pull
  *                through its memory path bounds these kernels, so for few weight rows an even
  *                deal over all CUs beats a fixed p1.  Up to 64 tokens, N/16 above the CU count and at
- *                most four times it; 16-bit weights with row-major B and C from one token block on,
+ *                most four times it (eight times with soft-FP8 weights, whose activations weigh twice as
+ *                much against the weight bytes); 16-bit weights with row-major B and C from one token block on,
  *                soft-FP8 weights or native B / C from 17 tokens on with p2 = 4 or 8 (the activations of
  *                a k window are then shared through LDS by the waves); otherwise the same as kernel 1
  *   kernel_id 5  kernel 3 with the K slices (p3) applied only to the panels that are left over after whole

@@ -35,7 +35,7 @@ What the columns select on gfx950 (the rows are produced by the scripts in
                                  kernelParam2 = 1: panels of 128 tokens, 2: of 256 tokens,
                                  other values: chosen from the shape)
                              4 = kernel 1 with one workgroup per CU and the row groups dealt out
-                                 evenly, two to four per workgroup (16-bit weights; soft-FP8 weights or
+                                 evenly, two to four per workgroup (16-bit weights; up to eight with soft-FP8 weights; soft-FP8 weights or
                                  layout-B activations from 17 tokens on with kernelParam2 = 4 or 8; row-major
                                  operands, up to 64 tokens, N/16 above the CU count; from 33 tokens on,
                                  and from 17 tokens on with kernelParam2 = 8, the activations of a k

@@ -589,9 +589,13 @@ static int launch_balanced(const GemmArgs &p, int wgs, hipStream_t s) {
         while (q.WK > 8) q.WK >>= 1;
         const int tiles_total = q.K / 32;
         while (q.WK >= 2 && tiles_total % q.WK != 0) q.WK >>= 1;
-        const size_t win_bytes = (size_t)2 * q.WK * stage_win_stride(CB) * 16;
-        size_t lds = (size_t)q.WK * RMAX * CB * 1024;
-        if (win_bytes > lds) lds = win_bytes;
+        auto lds_for = [](int wk) {
+            const size_t win_bytes = (size_t)2 * wk * stage_win_stride(CB) * 16, fold_bytes = (size_t)wk * RMAX * CB * 1024;
+            return win_bytes > fold_bytes ? win_bytes : fold_bytes;
+        };
+        // many row groups per workgroup: fewer waves, so that the fold of their partial sums still fits
+        while (q.WK > 2 && lds_for(q.WK) > 150 * 1024) q.WK >>= 1;
+        const size_t lds = lds_for(q.WK);
         if (q.WK < 2 || lds > 150 * 1024) return 1;      // does not apply: the caller falls back
         if constexpr (CB >= 2) {
             // more than 64 KiB of dynamic LDS has to be allowed once per kernel and device
@@ -610,21 +614,24 @@ static int launch_balanced(const GemmArgs &p, int wgs, hipStream_t s) {
         }
     }
     // soft-FP8 weights and layout-B activations take this kernel only with staged windows
-    if constexpr (FP8 || BMODE != MLK_B_ROWMAJOR) return 1;
-    while (q.WK * 64 > wave_kernel_threads(RMAX * CB, U, false) || (size_t)q.WK * RMAX * CB * 1024 > 64 * 1024) q.WK >>= 1;
-    size_t lds = q.WK > 1 ? (size_t)q.WK * RMAX * CB * 1024 : 0;
-    gemm_wave_balanced_kernel<T, CB, RMAX, U><<<wgs, q.WK * 64, lds, s>>>(q);
-    MLK_LAUNCH_CHECK();
-    return MLK_OK;
+    if constexpr (FP8 || BMODE != MLK_B_ROWMAJOR) {
+        return 1;
+    } else {
+        while (q.WK * 64 > wave_kernel_threads(RMAX * CB, U, false) || (size_t)q.WK * RMAX * CB * 1024 > 64 * 1024) q.WK >>= 1;
+        size_t lds = q.WK > 1 ? (size_t)q.WK * RMAX * CB * 1024 : 0;
+        gemm_wave_balanced_kernel<T, CB, RMAX, U><<<wgs, q.WK * 64, lds, s>>>(q);
+        MLK_LAUNCH_CHECK();
+        return MLK_OK;
+    }
 }
 
 // number of workgroups for kernel id 4 and the larger of the two row-group counts, or 0 when it does not apply
-static int balanced_grid(const GemmArgs &p, int CB, int *r_max) {
+static int balanced_grid(const GemmArgs &p, int CB, int *r_max, int most = 4) {
     const int cus = device_cus();
     const int groups = p.N / 16;
     if (groups <= cus) return 0;
     const int r = (groups + cus - 1) / cus;
-    if (r < 2 || r > 4 || CB > 4) return 0;
+    if (r < 2 || r > most || CB > 4) return 0;
     *r_max = r;
     return cus;
 }
@@ -654,7 +661,9 @@ static int launch_rc(const GemmArgs &p, int kernel_id, int R, int CB, hipStream_
     if constexpr (FP8 && BMODE == MLK_B_ROWMAJOR && CMODE == MLK_C_ROWMAJOR) {
         if (kernel_id == 4 && CB >= 2) {
             int r_max = 0;
-            const int wgs = p.SK == 1 ? balanced_grid(p, CB, &r_max) : 0;
+            // soft-FP8 weights are half the bytes per k tile, so the activations weigh twice as much against them:
+            // up to eight row groups per workgroup share one staged window (28672 rows: seven per workgroup)
+            const int wgs = p.SK == 1 ? balanced_grid(p, CB, &r_max, 8) : 0;
 #define MLK_BAL8(CC, RR)                                                  \
     if (wgs && CB == CC && r_max == RR) {                                 \
         const int rc = launch_balanced<T, CC, RR, true>(p, wgs, s);       \
@@ -663,6 +672,9 @@ static int launch_rc(const GemmArgs &p, int kernel_id, int R, int CB, hipStream_
             MLK_BAL8(2, 2) MLK_BAL8(2, 3) MLK_BAL8(2, 4)
             MLK_BAL8(3, 2) MLK_BAL8(3, 3) MLK_BAL8(3, 4)
             MLK_BAL8(4, 2) MLK_BAL8(4, 3) MLK_BAL8(4, 4)
+            MLK_BAL8(2, 5) MLK_BAL8(2, 6) MLK_BAL8(2, 7) MLK_BAL8(2, 8)
+            MLK_BAL8(3, 5) MLK_BAL8(3, 6) MLK_BAL8(3, 7) MLK_BAL8(3, 8)
+            MLK_BAL8(4, 5) MLK_BAL8(4, 6) MLK_BAL8(4, 7) MLK_BAL8(4, 8)
 #undef MLK_BAL8
         }
     }

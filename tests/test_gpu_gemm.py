@@ -280,12 +280,13 @@ def test_gemm_balanced_rows_kernel_shared_windows(mlk, dtype, k, m):
         assert torch.equal(c, c2)
 
 
-@pytest.mark.parametrize("n", [11008, 12288, 4736])
+@pytest.mark.parametrize("n", [11008, 12288, 4736, 18432, 22016, 28672, 32768])
 @pytest.mark.parametrize("m", [20, 32, 40, 64])
 def test_gemm_balanced_rows_kernel_soft_fp8(mlk, n, m):
-    """kernelId 4 with soft-FP8 weights from two token blocks on (eight waves share staged windows): three or two
-    row groups per workgroup that start anywhere, so they straddle two 128-row blocks of scales; every block has
-    its own random scale.  With two waves at two token blocks the id means kernel 1."""
+    """kernelId 4 with soft-FP8 weights from two token blocks on (eight waves share staged windows): two to eight
+    row groups per workgroup (on 256 CUs: three or two for 11008 rows, five or four for 18432, six or five for 22016,
+    seven for 28672, eight for 32768) that start anywhere, so they straddle two 128-row blocks of scales; every block
+    has its own random scale.  With two waves at two token blocks the id means kernel 1."""
     k = 1024
     codes = fp8_codes((n, k), 91)
     g = torch.Generator().manual_seed(92)
