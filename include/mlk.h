@@ -204,8 +204,9 @@ size_t mlk_gemm_counter_bytes(void);
  * 16 MiB per GPU, held until the process ends.  A call whose mlk_gemm_workspace_bytes(m, n, p1, p3) exceeds
  * that returns MLK_ERR_WORKSPACE and launches nothing.  The call allocates and frees nothing.  All calls on
  * one GPU share the array: calls that may overlap (different streams, or graphs replayed side by side) race;
- * order them on one stream.  The first call on a GPU looks up the array's address and clears the counter
- * region with a small kernel on `stream`. */
+ * order them on one stream.  The first call on a GPU looks up the array's address; nothing is cleared: the
+ * array is zero-filled when the library's code is loaded onto the GPU and every call leaves its arrival
+ * counters at zero again, so the call may be recorded into a HIP graph from the very first one on. */
 int mlk_gemm_layout_a_noalloc(const void *a, const void *b, void *c, int m, int n, int k, int a_kind, int x_kind,
                               int b_mode, int c_mode, float alpha, const void *bias, const float *scale,
                               int kernel_id, int p1, int p2, int p3, void *stream);
@@ -265,12 +266,16 @@ int mlk_fused_experts_compute(const void *w1, const void *w2, const void *x, int
                               void *stream);
 size_t mlk_moe_workspace_bytes(int n_tokens, int n_experts, int topk, int hidden, int inter);
 
-/* How mlk_fused_experts_compute would run one pass of min(n_tokens, 256) tokens, decided on the host from the
- * sizes alone (no GPU is touched): out[0] = kernel family (0 single-token GeMV kernels, 1 decode kernels that
- * align in-kernel, 2 decode kernels after the alignment kernel, 3 row-shared kernels), out[1] = token blocks
- * per task, out[2] = upper bound of the task list, out[3] = row groups per wave and out[4] = K slices of the
- * down projection, out[5] = waves and out[6] = dynamic LDS bytes of the decode down kernel (families 1, 2),
- * out[7] = its static LDS bytes.  For tests and the tuning scripts; no counterpart in the reference. */
+/* How mlk_fused_experts_compute would run one pass of min(n_tokens, 256) tokens; the launch code reads the same
+ * plan.  out[0] = kernel family (0 single-token GeMV kernels, 1 decode kernels that align in-kernel, 2 decode
+ * kernels after the alignment kernel, 3 row-shared kernels, 4 panel kernels: soft-FP8 weights with more than 64
+ * tokens per pass over an expert), out[1] = token blocks per task, out[2] = upper bound of the task list,
+ * out[3] = row groups per wave and out[4] = K slices of the down projection, out[5] = waves and out[6] = dynamic
+ * LDS bytes of the decode down kernel (families 1, 2), out[7] = its static LDS bytes.  Everything follows from
+ * the sizes alone except out[4] of family 4, which also depends on the number of compute units of the current
+ * device: for that family the call asks the HIP runtime for it (which initialises the runtime) and assumes 256
+ * where there is no GPU, so a plan made on a host without a GPU can name another slice count than a launch on a
+ * device with a different CU count uses.  For tests and the tuning scripts; no counterpart in the reference. */
 int mlk_moe_plan(int n_tokens, int n_experts, int topk, int hidden, int inter, int w_kind, int32_t *out);
 
 #ifdef __cplusplus

@@ -1,7 +1,8 @@
 """Build the C-ABI shared library `libmlk.so` for gfx950 with hipcc, in-tree.
 
 `python -m muxi_native_layout_kernels_amd.build` compiles every `csrc/*.hip`
-into one object each (in parallel) and links `muxi_native_layout_kernels_amd/libmlk.so`.
+into one object each (in parallel) and links `muxi_native_layout_kernels_amd/libmlk.so`;
+`python -m muxi_native_layout_kernels_amd.build mlk_moe mlk_gemv` recompiles only the named sources.
 hipcc cross-compiles, so no GPU is needed to build.
 """
 import os
@@ -38,10 +39,17 @@ def _compile(src):
     return obj
 
 
-def build(verbose=True):
+def build(verbose=True, only=None):
+    """Compile every source and link.  `only` (names of sources without the extension) recompiles just those and
+    links them with the objects a previous full build left in build/: for work on one kernel file."""
     srcs = sources()
-    with ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
-        objs = list(pool.map(_compile, srcs))
+    todo = srcs if not only else [s for s in srcs if os.path.basename(s)[:-4] in only]
+    with ThreadPoolExecutor(max_workers=min(8, max(1, len(todo)))) as pool:
+        list(pool.map(_compile, todo))
+    objs = [os.path.join(HERE, "build", os.path.basename(s)[:-4] + ".o") for s in srcs]
+    missing = [o for o in objs if not os.path.exists(o)]
+    if missing:
+        raise RuntimeError("no object for %s: run a full build first" % ", ".join(missing))
     cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *objs, "-o", OUT]
     proc = subprocess.run(cmd, capture_output=True, text=True)
     if proc.returncode != 0:
@@ -52,4 +60,4 @@ def build(verbose=True):
 
 
 if __name__ == "__main__":
-    build()
+    build(only=set(sys.argv[1:]) or None)

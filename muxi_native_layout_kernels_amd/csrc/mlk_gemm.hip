@@ -11,18 +11,18 @@ constexpr size_t kCounterBytes = 64 * 1024;
 
 // Scratch of mlk_gemm_layout_a_noalloc(): arrival counters and fp32 partials of the cross-workgroup K splits,
 // for callers that can neither allocate nor pass a workspace.  One copy per GPU, held until the process ends.
+// The array has no initialiser, so it is zero-filled when the code object is loaded onto a device, and the K-split
+// kernels leave every counter at zero again when a call ends (the last workgroup to arrive resets its counter):
+// nothing has to be cleared at set-up, and the first call may just as well be recorded into a HIP graph that is
+// replayed later or thrown away.  The partials need no clearing at all (every slice is written before it is read).
 constexpr size_t kStaticScratchBytes = (size_t)16 << 20;
 static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
 static std::atomic<void *> g_scratch_ptr[64];     // per device: the array's address on that device
 static std::mutex g_scratch_mutex;
 
-__global__ void __launch_bounds__(256) zero_words_kernel(uint32_t *p, int n) {
-    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) p[i] = 0u;
-}
-
-// Address of `scratch` on the current device.  On the first call on a device the address is looked up and
-// the counter region is cleared by a small kernel on `s` (ordered before the caller's launches on `s`).
-static int static_scratch(void **out, hipStream_t s) {
+// Address of `scratch` on the current device, looked up once per device (each GPU holds its own copy of the
+// array at its own address).  Host code uses this pointer, never the array's name.
+static int static_scratch(void **out) {
     int dev = 0;
     hipError_t e = hipGetDevice(&dev);
     if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));
@@ -35,9 +35,6 @@ static int static_scratch(void **out, hipStream_t s) {
             e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
             if (e != hipSuccess || ptr == nullptr)
                 return fail(MLK_ERR_LAUNCH, e != hipSuccess ? hipGetErrorString(e) : "gemm: no address for the static scratch");
-            zero_words_kernel<<<16, 256, 0, s>>>((uint32_t *)ptr, (int)(kCounterBytes / 4));
-            e = hipGetLastError();
-            if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));
             g_scratch_ptr[dev].store(ptr, std::memory_order_release);
         }
     }
@@ -186,7 +183,7 @@ extern "C" int mlk_gemm_layout_a_noalloc(const void *a, const void *b, void *c, 
             return fail(MLK_ERR_WORKSPACE,
                         "gemm: this K split needs more than the 16 MiB of built-in scratch; use fewer splits (p3) "
                         "or mlk_gemm_layout_a with a caller-owned workspace");
-        const int rc = static_scratch(&ws, (hipStream_t)stream);
+        const int rc = static_scratch(&ws);
         if (rc != MLK_OK) return rc;
     }
     return mlk_gemm_layout_a(a, b, c, m, n, k, a_kind, x_kind, b_mode, c_mode, alpha, bias, scale, kernel_id, p1, p2,

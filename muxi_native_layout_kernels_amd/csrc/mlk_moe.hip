@@ -1134,9 +1134,11 @@ struct MoeWorkspace {
     int sb;          // token blocks the intermediate is dimensioned for
 };
 
-constexpr int kDecodeKSlices = 4;
-
 static inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
+
+// Bytes of the fp32 buffer that holds the K-sliced down projections of one pass of tc tokens (defined below the
+// plan it reads).
+static size_t moe_obuf_bytes(int tc, int n_experts, int topk, int hidden, int inter);
 
 static size_t carve(uint8_t *base, int tc, int E, int K, int hidden, int inter, MoeWorkspace *ws) {
     const int n_pairs = tc * K;
@@ -1159,10 +1161,8 @@ static size_t carve(uint8_t *base, int tc, int E, int K, int hidden, int inter, 
     // seven spare blocks: the row-shared down kernel always fetches CB <= 8 consecutive blocks
     w.sb = max_blocks + 7;
     w.hbuf = (uint16_t *)take((size_t)inter * w.sb * 16 * 2);
-    // fp32 buffer of the K-sliced down projections: per routed pair and slice for the row-shared
-    // kernels, per token and slice (up to 4) for the decode kernel
-    w.obuf = (float *)take(tc > 16 ? (size_t)n_pairs * 8 * hidden * sizeof(float)
-                                   : (size_t)tc * kDecodeKSlices * hidden * sizeof(float));   // 8 = kMoeMaxKSlices
+    // fp32 buffer of the K-sliced down projections, sized for the slices the plan of this pass really uses
+    w.obuf = (float *)take(moe_obuf_bytes(tc, E, K, hidden, inter));
     w.counters = (int32_t *)take(sizeof(int32_t) * (size_t)(hidden / 16));
     if (ws) *ws = w;
     return off;
@@ -1233,7 +1233,7 @@ static int launch_moe(const MoeArgs &a, int max_tasks, hipStream_t s) {
     return launch_moe_down<T, FP8, CB, 1, INLINE>(a, 1, s);
 }
 
-constexpr int kMoeMaxKSlices = 8;  // K slices of the row-shared down projection (sizes its fp32 buffer)
+constexpr int kMoeMaxKSlices = 8;  // most K slices of the row-shared and panel down projections
 
 // Row groups per wave and K slices of the row-shared down projection for CB token blocks per task.
 static int moe_tile_down_rows(int cb, int H) {
@@ -1350,6 +1350,23 @@ static MoePlan moe_plan(int tc, int n_experts, int topk, int hidden, int inter, 
     return pl;
 }
 
+// Per routed pair and slice for the row-shared and panel kernels, per token and slice for the decode kernels,
+// nothing for the single-token kernels; the larger of the two weight kinds, since the workspace query does not
+// know which one the call will bring.
+static size_t moe_obuf_bytes(int tc, int n_experts, int topk, int hidden, int inter) {
+    size_t bytes = 256;
+    for (int fp8 = 0; fp8 < 2; ++fp8) {
+        const MoePlan pl = moe_plan(tc, n_experts, topk, hidden, inter, fp8 != 0);
+        size_t need = 0;
+        if (pl.path == kMoePathTile || pl.path == kMoePathPanel)
+            need = (size_t)tc * topk * pl.down_slices * hidden * sizeof(float);
+        else if (pl.path != kMoePathGemv1)
+            need = (size_t)tc * pl.down_slices * hidden * sizeof(float);
+        if (need > bytes) bytes = need;
+    }
+    return bytes;
+}
+
 }  // namespace mlk
 
 using namespace mlk;
@@ -1420,8 +1437,16 @@ extern "C" int mlk_moe_align_tokens(const int32_t *topk_ids, int n_pairs, int n_
 }
 
 extern "C" size_t mlk_moe_workspace_bytes(int n_tokens, int n_experts, int topk, int hidden, int inter) {
-    int tc = n_tokens < kMoeChunk ? n_tokens : kMoeChunk;
-    return carve(nullptr, tc, n_experts, topk, hidden, inter, nullptr);
+    // the passes of a call share the workspace: full passes of kMoeChunk tokens and a shorter last one, whose plan
+    // (more K slices over fewer pairs) may ask for a different carving
+    const int tc = n_tokens < kMoeChunk ? n_tokens : kMoeChunk;
+    size_t bytes = carve(nullptr, tc, n_experts, topk, hidden, inter, nullptr);
+    const int last = n_tokens > kMoeChunk ? n_tokens % kMoeChunk : 0;
+    if (last > 0) {
+        const size_t b2 = carve(nullptr, last, n_experts, topk, hidden, inter, nullptr);
+        if (b2 > bytes) bytes = b2;
+    }
+    return bytes;
 }
 
 extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const void *x, int n_tokens, int n_experts,

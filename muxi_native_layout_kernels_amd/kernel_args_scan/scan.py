@@ -175,9 +175,19 @@ def _copies(nbytes):
     return int(max(2, min(16, (3 * MALL_BYTES + nbytes - 1) // nbytes)))
 
 
-def _gate(got, want):
+GATE_FAILURES = []      # configurations that ran and gave a wrong result: a bug to report, not a slow candidate
+
+
+def _gate(got, want, what=None):
+    """True when `got` matches the fp32 product within rtol = atol = 1e-2.  A configuration that ran but fails is
+    named on stderr and remembered: main() exits non-zero if there was any, so a kernel path that computes wrong
+    results for some shape shows up instead of silently dropping out of the tables."""
     err = (got.float() - want).abs()
-    return bool((err <= 1e-2 + 1e-2 * want.abs()).all())
+    ok = bool((err <= 1e-2 + 1e-2 * want.abs()).all())
+    if not ok and what is not None:
+        GATE_FAILURES.append(what)
+        print("WRONG RESULT (max error %g): %s" % (float(err.max()), what), file=sys.stderr, flush=True)
+    return ok
 
 
 def scan_gemv(table, shapes, iters, progress=None):
@@ -204,7 +214,7 @@ def scan_gemv(table, shapes, iters, progress=None):
             def call(a):
                 return lambda: ops.gemv_layoutA_wapper(a, x, n, k, 1, 0, block, kid, p1, p2, scale, None)
             try:
-                if not _gate(call(packed[0])(), want):
+                if not _gate(call(packed[0])(), want, "%s %dx%d BLOCK_DIM_X=%d kernelId=%d p1=%d p2=%d" % (table, n, k, block, kid, p1, p2)):
                     continue
             except RuntimeError:                             # a configuration the library rejects for this shape
                 continue
@@ -287,7 +297,7 @@ def scan_gemm(table, shapes, tokens, iters, progress=None, known=(), kernel_ids=
                         continue
                     if mode == "native":
                         got = ops.reLayoutC(got)
-                    if not _gate(got, want):
+                    if not _gate(got, want, "%s %dx%d M=%d kernelId=%d p1=%d p2=%d p3=%d" % (table, n, k, m, kid, p1, p2, p3)):
                         continue
                     us = _time_graph([call(a) for a in packed], iters)
                     if best is None or us < best[0]:
@@ -342,6 +352,9 @@ def main():
             rows = scan_gemm(table, shapes, tokens, args.iters, progress, known, ids)
         out.close()
         print("wrote %d rows to %s" % (len(rows), path), file=sys.stderr)
+    if GATE_FAILURES:
+        print("%d configurations ran but gave wrong results (listed above)" % len(GATE_FAILURES), file=sys.stderr)
+        sys.exit(2)
 
 
 if __name__ == "__main__":

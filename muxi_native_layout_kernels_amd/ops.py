@@ -84,9 +84,39 @@ class WorkspacePool:
         with self._lock:
             return list(self._live.values()) + list(self._retired)
 
+    def held_bytes(self):
+        with self._lock:
+            return sum(b.numel() for b in self._live.values()) + sum(b.numel() for b in self._retired)
+
+    def release(self, retired_only=False):
+        """Drop the retired buffers and, unless `retired_only`, the live ones too (they are re-created on the next
+        call).  Only for callers that hold no captured graph which replays one of these pointers, and with no call
+        of this library in flight on the device."""
+        with self._lock:
+            freed = sum(b.numel() for b in self._retired)
+            self._retired = []
+            if not retired_only:
+                freed += sum(b.numel() for b in self._live.values())
+                self._live = {}
+        return freed
+
 
 _gemm_pool = WorkspacePool(1 << 22, zero_prefix=True)
 _moe_pool = WorkspacePool(1 << 20)
+
+
+def workspace_bytes_held():
+    """Device bytes the library's scratch pools hold right now (K-split partials, MoE tables and intermediates)."""
+    return _gemm_pool.held_bytes() + _moe_pool.held_bytes()
+
+
+def release_workspaces(retired_only=False):
+    """Give the scratch memory of the K-split GeMMs and of the fused MoE back to torch's allocator and return the
+    number of bytes released.  The pools keep one buffer per (device, stream) and never free by themselves, so that
+    a HIP graph captured around a call replays with valid pointers; a caller that holds no such graph (or has
+    dropped it) calls this after a burst of large batches, or when streams it used are gone.  `retired_only`
+    releases just the buffers that a larger one has replaced.  Synchronize the device first."""
+    return _gemm_pool.release(retired_only) + _moe_pool.release(retired_only)
 
 
 def _workspace(device, nbytes, counter_bytes, stream=None):
@@ -571,5 +601,5 @@ __all__ = [
     "gemm_layoutA_soft_fp8_wapper", "gemm_layoutAB_ContinuousC_wapper", "gemv_layoutA_wapper", "fp8_weight_repack",
     "routing_gate", "experts_compute", "fused_routing_gate",
     "batched_routed_activation_indexed_to_expert_block_indexed", "fused_experts_compute",
-    "pack_layout_a", "unpack_layout_a", "experts_compute_raw",
+    "pack_layout_a", "unpack_layout_a", "experts_compute_raw", "release_workspaces", "workspace_bytes_held",
 ]

@@ -406,17 +406,24 @@ def test_gemm_soft_fp8(mlk, m, scaled):
 
 
 @pytest.mark.parametrize("m", [4, 16])
-def test_gemm_soft_fp8_config(mlk, m):
+@pytest.mark.parametrize("scaled", [False, True])
+def test_gemm_soft_fp8_config(mlk, m, scaled):
+    """The third benchmark configuration at its full shape through the shipped table rows, with unit scales and
+    with an arbitrary fp32 scale per 128 x 128 block (the general widening path, which is what the bench times)."""
     n, k = 28672, 8192
     codes = fp8_codes((n, k), 2025)
     b = randn((m, k), torch.bfloat16, 1.0, 2026)
-    scale = torch.ones((n // 128, k // 128))
+    if scaled:
+        g = torch.Generator().manual_seed(2027)
+        scale = (torch.rand((n // 128, k // 128), generator=g) * 0.02 + 0.001).float()
+    else:
+        scale = torch.ones((n // 128, k // 128))
     c = mlk.gemm_layoutA_soft_fp8(pack_a(codes).cuda(), scale.cuda(), b.cuda())
     # float64 product in row chunks to bound host memory
     from oracle import softfp8
     got = c.cpu()
     for r0 in range(0, n, 4096):
-        wchunk = softfp8.dequant_weight_f32(codes[r0:r0 + 4096].numpy(), None)
+        wchunk = softfp8.dequant_weight_f32(codes[r0:r0 + 4096].numpy(), scale[r0 // 128:(r0 + 4096) // 128].numpy() if scaled else None)
         assert_close(got[:, r0:r0 + 4096], ogemm.linear_expected(wchunk, b), RTOL, ATOL, "soft-fp8 config")
 
 

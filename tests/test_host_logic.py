@@ -117,6 +117,40 @@ def test_workspace_pool_never_frees_what_it_handed_out():
     assert len(pool.owned()) <= 8
 
 
+def test_workspace_pool_release():
+    """release() drops the retired buffers (and the live ones unless asked not to) and says how much that was;
+    the next request simply gets a new buffer."""
+    pool = ops.WorkspacePool(1024)
+    cpu = torch.device("cpu")
+    a = pool.get(cpu, 0, 1000)
+    b = pool.get(cpu, 0, 1 << 16)                             # retires a
+    assert pool.held_bytes() == a.numel() + b.numel()
+    assert pool.release(retired_only=True) == a.numel() and pool.held_bytes() == b.numel()
+    assert pool.get(cpu, 0, 100) is b                         # the live buffer is still the one in use
+    assert pool.release() == b.numel() and pool.held_bytes() == 0
+    c = pool.get(cpu, 0, 100)
+    assert c is not b and c.numel() >= 1024
+
+
+def test_moe_workspace_follows_the_plan():
+    """The fp32 buffer of the K-sliced down projections is sized for the slices the plan uses (not for the most
+    the kernels could take), a call of several passes covers its shorter last pass, and the query grows with the
+    token count within a pass."""
+    lib = _lib.load()
+    E, K, H, I = 256, 8, 7168, 2048
+    sizes = [lib.mlk_moe_workspace_bytes(t, E, K, H, I) for t in (1, 16, 64, 256)]
+    assert sizes == sorted(sizes)
+    # 256 tokens: 2048 pairs; eight slices of fp32 rows would be 470 MB, the plan uses far fewer
+    slices = max(_plan(256, E, K, H, I, kind)["down_slices"] for kind in (1, 2))
+    assert sizes[-1] < 2048 * H * 4 * (slices + 1) + (64 << 20)
+    for n in (257, 300, 500, 511, 1024):
+        last = n % 256
+        need = lib.mlk_moe_workspace_bytes(n, E, K, H, I)
+        assert need >= lib.mlk_moe_workspace_bytes(256, E, K, H, I)
+        if last:
+            assert need >= lib.mlk_moe_workspace_bytes(last, E, K, H, I)
+
+
 def test_routing_buffers_are_kept_for_every_shape_and_stream():
     from muxi_native_layout_kernels_amd import moe_planC
     cpu = torch.device("cpu")

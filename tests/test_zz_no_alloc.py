@@ -81,3 +81,32 @@ def test_noalloc_rejects_what_exceeds_the_built_in_scratch(mlk):
     rc = lib.mlk_gemm_layout_a_noalloc(x.data_ptr(), x.data_ptr(), x.data_ptr(), 64, 28672, 8192, 1, 1, 0, 0, 1.0, None,
                                        None, 1, 1, 4, 8, torch.cuda.current_stream().cuda_stream)
     assert rc == -3 and b"16 MiB" in lib.mlk_last_error()
+
+
+def test_noalloc_recorded_into_a_graph_and_replayed(mlk):
+    """The call recorded into a HIP graph with a K split across workgroups (so the built-in scratch is in use),
+    replayed twice with eager work and synchronizations in between: every replay must give the workspace
+    variant's bits, and the replays must leave the arrival counters clean for the eager call that follows."""
+    lib = _lib()
+    w = randn((2048, 4096), torch.bfloat16, 0.02, 31)
+    b = randn((32, 4096), torch.bfloat16, 1.0, 32)
+    n, k, m = 2048, 4096, 32
+    a, bd = pack_a(w).cuda(), b.cuda()
+    _, want = _both(lib, w, b, 1, 2, 4, 4)
+    out = torch.zeros((m, n), dtype=torch.bfloat16, device="cuda")
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        with torch.cuda.graph(graph, stream=stream):
+            rc = lib.mlk_gemm_layout_a_noalloc(a.data_ptr(), bd.data_ptr(), out.data_ptr(), m, n, k, 1, 1, 0, 0, 1.0, None,
+                                               None, 1, 2, 4, 4, torch.cuda.current_stream().cuda_stream)
+            assert rc == 0, lib.mlk_last_error()
+        for _ in range(2):
+            out.zero_()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(out, want)
+            # eager work of the program between the replays
+            c0, c1 = _both(lib, w, b, 1, 2, 4, 4)
+            assert torch.equal(c0, c1) and torch.equal(c0, want)
