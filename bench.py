@@ -2,6 +2,7 @@
 """Benchmark of the native-layout hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--quick] [--case TEXT] [--no-cpu] [--case-steps S]
+                    [--no-eager] [--no-blas] [--counters]
 
 Prints ONE JSON line.  The headline workload is the fp16 narrow GeMM of the
 second benchmark configuration (`gemm_layoutA`, weights 11008 x 4096 in
@@ -39,6 +40,15 @@ where the weights are small, HBM traffic from hardware counters where a
 profile under profiles/ holds it, and the CPU baseline of that configuration:
 the reference's CPU-runnable torch path (a library linear on the un-packed
 weights, or its dense MoE loop) timed on the host cores on a bounded sample.
+
+`eager_calls` holds the public Python API timed the way the reference's own
+scripts time it: the wall clock around 1000 eager calls (300 for the fused MoE),
+synchronized at both ends, host work included, next to the device time per
+call of the same configuration.
+
+`--counters` is for runs under `rocprofv3 --pmc`: every call is launched
+directly, a handful per case, and no HIP graph is built (counter collection
+over graph replays with thousands of dispatches crashed the profiler).
 """
 import argparse
 import json
@@ -71,12 +81,21 @@ def main():
     ap.add_argument("--case", default=None,
                     help="besides the headline, run only the per-configuration cases whose name contains this text "
                          "(several texts separated by commas; for profiling single kernels)")
+    ap.add_argument("--counters", action="store_true",
+                    help="for runs under a hardware-counter profiler: every call is launched directly (no HIP graph is "
+                         "built or replayed: counter collection over graph replays with thousands of dispatches has "
+                         "crashed the profiler), no settle replays, --steps calls per case after --warmup calls, no "
+                         "yardsticks, no vendor BLAS, no CPU legs, no eager-call lines; the headline runs only if "
+                         "--case names it; timings of such a run are not benchmark numbers")
+    ap.add_argument("--no-eager", action="store_true", help="skip the eager-call lines (public Python API, wall clock)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain copy kernel of known size (256 MiB in, 256 MiB out) so that "
                          "hardware byte counters can be scaled against it")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
+    if args.counters:
+        args.no_cpu = args.no_blas = args.no_eager = True
 
     import torch
     if not torch.cuda.is_available():
@@ -136,6 +155,23 @@ def main():
         the median over the runs (`us`), the first run and the minimum, and the host-clock seconds of one more replay
         of the graph between two synchronizations."""
         stream = bench_stream
+        if args.counters:
+            with torch.cuda.stream(stream):
+                for i in range(min(warmup, 3)):
+                    calls[i % len(calls)]()
+                torch.cuda.synchronize()
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                n = min(steps, 8)
+                t0 = time.perf_counter()
+                e0.record()
+                for i in range(n):
+                    calls[i % len(calls)]()
+                e1.record()
+                torch.cuda.synchronize()
+                wall = time.perf_counter() - t0
+            us = e0.elapsed_time(e1) * 1e3 / n
+            return dict(us=us, us_first=us, us_median=us, us_min=us, wall=wall * steps / n,
+                        how="counter run: %d direct launches, no graph" % n)
         with torch.cuda.stream(stream):
             for i in range(max(warmup, 3)):
                 calls[i % len(calls)]()
@@ -179,8 +215,12 @@ def main():
                    gbps=algo / t["us"] / 1e3, frac=algo / t["us"] / 1e3 / HBM_PEAK_GBPS, wall=t["wall"], how=t["how"])
         row.update(extra)
         got = traffic_table.get(name)
-        if isinstance(got, dict):   # counted for one routing: valid only when this run drew as many active experts
-            got = got["bytes"] if got.get("active_experts") == extra.get("active_experts") else None
+        if isinstance(got, dict):
+            # counted for one routing / one set of launch parameters: valid only for a run that has the same
+            ok = got.get("active_experts") == extra.get("active_experts") if "active_experts" in got else True
+            if "params" in got and list(got["params"]) != list(extra.get("params") or []):
+                ok = False
+            got = got["bytes"] if ok else None
         if got is not None:
             row["traffic"] = got
             row["traffic_over_algorithmic"] = got / algo
@@ -295,7 +335,7 @@ def main():
         algo = wbytes + (scale.numel() * 4 if scale is not None else 0) + k * 2 + n * 2
         extra = dict(params=[block, kid, p1, p2], copies=len(A))
         del A
-        if yardstick:
+        if yardstick and not args.counters:
             extra["read_only_us"] = read_only_us(wbytes, steps)
         if cpu_rows:
             extra["cpu_baseline"] = cpu_linear(n, k, 1, kind, cpu_rows)
@@ -312,7 +352,8 @@ def main():
                             % (count, str(dt).replace("torch.", "")))
         del W
 
-    def gemm_case(name, n, k, kind, m, steps, warmup, native=False, copies=None, cpu_rows=2048, cpu=True, blas=False):
+    def gemm_case(name, n, k, kind, m, steps, warmup, native=False, copies=None, cpu_rows=2048, cpu=True, blas=False,
+                  relayout=True):
         xk = 1 if kind == 2 else kind
         A = weights(n, k, kind, copies or copies_for(n * k * (1 if kind == 2 else 2)))
         b = torch.randn((m, k), generator=gen, device=dev).to(DT[xk])
@@ -339,12 +380,12 @@ def main():
                                                  0 if scale is None else scale.data_ptr(), kid, p1, p2, p3, ws_ptr, ws_len,
                                                  st),
                            "gemm")
-                if native:
+                if native and relayout:
                     _lib.check(lib.mlk_re_layout_c(c.data_ptr(), c_rm.data_ptr(), m, n, st), "reLayoutC")
             return call
         t = run_graph([mk(a) for a in A], steps, warmup, direct_if_short=True)
         algo = n * k * (1 if kind == 2 else 2) + (scale.numel() * 4 if scale is not None else 0) + m * k * 2 + m * n * 2
-        if native:
+        if native and relayout:
             algo += 2 * m * n * 2
         row = finish(name, t, algo, params=[kid, p1, p2, p3], copies=len(A))
         if cpu:
@@ -490,6 +531,81 @@ def main():
         t = run_graph([mk(a) for a in src], steps, 3)
         return finish(name, t, 2 * e * n * k * 2)
 
+    def eager_case(name, make, calls=1000, warm=1000):
+        """The public Python API called eagerly, the way the reference's scripts time it
+        (benchmark_and_test/gemv_benchmark.py:62-73, benchmark_muxi_moe.py:40-49): `warm` calls, a synchronization,
+        then the wall clock around `calls` back-to-back calls with one synchronization at the end.  Host work per call
+        (argument checks, table lookup, output allocation, the ctypes call, the launch) is part of it; `graph_us`
+        beside it is the same configuration's device time per call from the graph-replay timing.  `make` returns
+        (call, name of the per_config line that holds the device time, or None for the headline)."""
+        call, ref = make()
+        with torch.cuda.stream(bench_stream):
+            for _ in range(warm):
+                call()
+            torch.cuda.synchronize()
+            runs = []
+            for _ in range(3):
+                t0 = time.perf_counter()
+                for _ in range(calls):
+                    call()
+                torch.cuda.synchronize()
+                runs.append((time.perf_counter() - t0) * 1e6 / calls)
+            # host cost alone: the same calls with nothing waiting on the device (queue drained first, clock stopped
+            # before the synchronization)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(200):
+                call()
+            host = (time.perf_counter() - t0) * 1e6 / 200
+            torch.cuda.synchronize()
+        row = dict(name=name, eager_us=round(statistics.median(runs), 3), eager_us_min=round(min(runs), 3),
+                   host_us_per_call=round(host, 3), calls=calls,
+                   how="wall clock around %d eager calls of the public Python API, synchronized at both ends; median of 3" % calls)
+        dev = head["us"] if ref is None else next((r["us"] for r in per_config if r["name"] == ref), None)
+        if dev is not None:
+            row["graph_us"] = round(dev, 3)
+            row["eager_over_graph"] = round(row["eager_us"] / dev, 3)
+        return row
+
+    def eager_gemv(n, k, kind, ref):
+        def make():
+            xk = 1 if kind == 2 else kind
+            a = weights(n, k, kind, copies_for(n * k * (1 if kind == 2 else 2)))
+            x = torch.randn((1, k), generator=gen, device=dev).to(DT[xk])
+            scale = block_scales(((n + 127) // 128, (k + 127) // 128)) if kind == 2 else None
+            state = {"i": 0}
+
+            def call():
+                state["i"] = (state["i"] + 1) % len(a)
+                return mlk.gemv_layoutA(a[state["i"]], x, scale_matrix=scale)
+            return call, ref
+        return make
+
+    def eager_gemm(n, k, kind, m, ref):
+        def make():
+            a = weights(n, k, kind, copies_for(n * k * 2))
+            b = torch.randn((m, k), generator=gen, device=dev).to(DT[kind])
+            state = {"i": 0}
+
+            def call():
+                state["i"] = (state["i"] + 1) % len(a)
+                return mlk.gemm_layoutA(a[state["i"]], b)
+            return call, ref
+        return make
+
+    def eager_moe(T, fp8, ref):
+        def make():
+            E, K, H, I = 8, 2, 4096, 14336
+            key = "fp8" if fp8 else "bf16"
+            if key not in moe_w:
+                moe_case("(weights for the eager line)", T, fp8, 2, 1)     # draws and caches the expert weights
+            w1, w2, s1, s2 = moe_w[key]
+            x = torch.randn((T, H), generator=gen, device=dev).to(torch.bfloat16)
+            logits = torch.randn((T, E), generator=gen, device=dev).to(torch.bfloat16)
+            kw = dict(w1_scale=s1, w2_scale=s2, block_shape=[128, 128], soft_fp8=True) if fp8 else {}
+            return (lambda: fused_moe(x, w1, w2, logits, K, True, **kw)), ref
+        return make
+
     if args.calibrate_copy:
         src = torch.randint(0, 255, (256 << 20,), dtype=torch.uint8, device=dev)
         dst = torch.empty_like(src)
@@ -516,8 +632,15 @@ def main():
     # ------------------------------------------------------------ headline
     N, K_, M = 11008, 4096, 16
     HEAD = "C2 fp16 gemm_layoutA 11008x4096 M=16"
-    head = gemm_case(HEAD, N, K_, 0, M, args.steps, args.warmup, blas=not args.quick)
+    head_wanted = not args.counters or (args.case is not None and any(part and part in HEAD for part in args.case.split(",")))
+    if head_wanted:
+        head = gemm_case(HEAD, N, K_, 0, M, args.steps, args.warmup, blas=not args.quick, cpu=not args.counters)
+    else:       # a counter run on other cases: no headline launches among the profiled dispatches
+        head = dict(name=HEAD, us=0.0, us_first=0.0, us_median=0.0, us_min=0.0,
+                    gbps=0.0, frac=0.0, wall=0.0, how="not run (--counters without the headline in --case)",
+                    bytes=N * K_ * 2 + M * K_ * 2 + M * N * 2, copies=0, params=None)
     per_config = []
+    eager = []
 
     def add(case, name, *a, **kw):
         """Run one per-configuration case unless --case asks for others only."""
@@ -526,17 +649,26 @@ def main():
     ceiling = None
     resident = None
     same_size = None
+    def add_eager(name, make, **kw):
+        if not args.no_eager and (args.case is None or any(part and part in name for part in args.case.split(","))):
+            eager.append(eager_case(name, make, **kw))
     if not args.quick:
-        one = gemm_case("headline workload, one weight copy (stays in the 256 MiB Infinity Cache)", N, K_, 0, M, args.steps,
-                        args.warmup, copies=1, cpu=False)
-        resident = {"us_per_call": round(one["us"], 3), "gbps": round(one["gbps"], 1),
-                    "what": "same kernel and launch parameters on a single 86 MiB weight copy: the stream comes from "
-                            "the Infinity Cache, not HBM; reported for information, never the headline"}
-        ceiling = round(read_ceiling(40), 1)
-        # the same yardstick at the headline's size: one launch that only reads as many bytes as the weights hold
-        same_size = read_only_us(N * K_ * 2, args.steps)
-        short = max(20, min(args.steps, args.case_steps))
+        if not args.counters:
+            one = gemm_case("headline workload, one weight copy (stays in the 256 MiB Infinity Cache)", N, K_, 0, M,
+                            args.steps, args.warmup, copies=1, cpu=False)
+            resident = {"us_per_call": round(one["us"], 3), "gbps": round(one["gbps"], 1),
+                        "what": "same kernel and launch parameters on a single 86 MiB weight copy: the stream comes from "
+                                "the Infinity Cache, not HBM; reported for information, never the headline"}
+            ceiling = round(read_ceiling(40), 1)
+            # the same yardstick at the headline's size: one launch that only reads as many bytes as the weights hold
+            same_size = read_only_us(N * K_ * 2, args.steps)
+        short = max(20, min(args.steps, args.case_steps)) if not args.counters else args.steps
         add(gemv_case, "C1 bf16 gemv 4096x4096", 4096, 4096, 1, short, 10, yardstick=True, cpu_rows=4096)
+        # the same GeMV on larger squares (the target speaks of N = K >= 4096), each with its own read-only yardstick
+        add(gemv_case, "C1+ bf16 gemv 8192x8192", 8192, 8192, 1, short, 10, yardstick=True, cpu_rows=0)
+        add(gemv_case, "C1+ bf16 gemv 16384x16384", 16384, 16384, 1, max(20, short // 4), 10, yardstick=True, cpu_rows=0)
+        add_eager("eager: gemv_layoutA bf16 4096x4096", eager_gemv(4096, 4096, 1, "C1 bf16 gemv 4096x4096"))
+        add_eager("eager: gemm_layoutA fp16 11008x4096 M=16", eager_gemm(N, K_, 0, M, None))
         for m in (1, 8, 32, 64):
             add(gemm_case, "C2 fp16 gemm_layoutA 11008x4096 M=%d" % m, N, K_, 0, m, short, 10, blas=True)
         add(gemv_case, "C2 fp16 gemv 11008x4096", N, K_, 0, short, 10)
@@ -545,15 +677,24 @@ def main():
             unit_scales=True)
         for m in (4, 16):
             add(gemm_case, "C3 soft-fp8 gemm_layoutA 28672x8192 M=%d" % m, 28672, 8192, 2, m, short, 10, cpu_rows=1024)
+        add_eager("eager: gemv_layoutA soft-fp8 28672x8192", eager_gemv(28672, 8192, 2, "C3 soft-fp8 gemv 28672x8192"))
         add(gemm_case, "C4 bf16 gemm_layoutABC+reLayoutC 8192x8192 M=32", 8192, 8192, 1, 32, short, 10, native=True,
             cpu_rows=1024, blas=True)
+        # the product alone, output left in layout-C as a following native-layout product would take it
+        add(gemm_case, "C4 bf16 gemm_layoutABC 8192x8192 M=32, output kept in layout-C", 8192, 8192, 1, 32, short, 10,
+            native=True, cpu=False, relayout=False)
         add(relayout_case, "C4 layoutB bf16 [32, 8192]", "layoutB", short)
         add(relayout_case, "C4 reLayoutC bf16 [32, 8192]", "reLayoutC", short)
         add(relayout_case, "C3 fp8_weight_repack 28672x8192", "fp8_weight_repack", 10)
         for T in (1, 16, 64, 256):
             add(moe_case, "C5 bf16 fused_moe T=%d" % T, T, False, args.moe_steps, 5)
+        for T in (1, 16):
+            add_eager("eager: fused_moe bf16 T=%d" % T, eager_moe(T, False, "C5 bf16 fused_moe T=%d" % T), calls=300, warm=100)
         for T in (1, 16, 64, 256):
             add(moe_case, "C5 soft-fp8 fused_moe T=%d" % T, T, True, args.moe_steps, 5)
+        for T in (1, 16):
+            add_eager("eager: fused_moe soft-fp8 T=%d" % T, eager_moe(T, True, "C5 soft-fp8 fused_moe T=%d" % T), calls=300,
+                      warm=100)
         for T in (1, 16):
             add(moe_next_case, "next: grouped-routing MoE E=256 top-8 H=7168 I=2048 bf16 T=%d" % T, T, args.moe_steps, 5)
         moe_w.clear()
@@ -597,7 +738,7 @@ def main():
                    "launch_params": head["params"],
                    "algorithmic_bytes": head["bytes"]},
         "roofline": {"bound": "hbm", "achieved": round(head["gbps"], 2), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(head["frac"], 4), "traffic": traffic_table.get(HEAD)},
+                     "frac": round(head["frac"], 4), "traffic": head.get("traffic")},
         "hbm_read_ceiling": None if ceiling is None else {
             "value": ceiling, "unit": "GB/s",
             "what": "pure streaming read (mlk_stream_read, 256 MiB x 4 rotating buffers) measured in this run",
@@ -606,6 +747,7 @@ def main():
         "vendor_blas": None if head.get("blas_us") is None else {
             "us_per_call": round(head["blas_us"], 3), "what": head["blas_note"] + ", same token count, same graph-replay timing"},
         "cpu_baseline": head.get("cpu_baseline"),
+        "eager_calls": eager,
         "per_config": per_config,
     }
     print(json.dumps(line))
