@@ -88,6 +88,8 @@ def main():
                          "yardsticks, no vendor BLAS, no CPU legs, no eager-call lines; the headline runs only if "
                          "--case names it; timings of such a run are not benchmark numbers")
     ap.add_argument("--no-eager", action="store_true", help="skip the eager-call lines (public Python API, wall clock)")
+    ap.add_argument("--tunable", action="append", default=[], metavar="ID=VALUE",
+                    help="set an experiment switch of the library (mlk_set_tunable) before anything runs; repeatable")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain copy kernel of known size (256 MiB in, 256 MiB out) so that "
                          "hardware byte counters can be scaled against it")
@@ -104,6 +106,9 @@ def main():
     from muxi_native_layout_kernels_amd import _lib, arg_selector
     from muxi_native_layout_kernels_amd.moe_planC import fused_moe
     lib = _lib.load()
+    for item in args.tunable:
+        ident, value = item.split("=")
+        lib.mlk_set_tunable(int(ident), int(value))
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     gen = torch.Generator(device=dev).manual_seed(2025)

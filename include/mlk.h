@@ -266,6 +266,19 @@ int mlk_fused_experts_compute(const void *w1, const void *w2, const void *x, int
                               void *stream);
 size_t mlk_moe_workspace_bytes(int n_tokens, int n_experts, int topk, int hidden, int inter);
 
+/* The whole MoE layer in one call: router, alignment, both grouped GeMMs, weighted sum.  Replaces the call
+ * sequence of the reference's Python entry `muxi_moe_planC.fused_moe` (muxi_layout_kernels/muxi_moe_planC.py:44-146:
+ * `fused_routing_gate`, the renormalisation in torch, the workspace fills, `fused_experts_compute`).  Arguments
+ * as for mlk_fused_routing_gate (logits [T, n_router_experts]; ids / weights are outputs, [T, K]) and
+ * mlk_fused_experts_compute (n_experts = expert slabs held locally; differs from n_router_experts only under an
+ * experts_map).  Same launches and results as the two calls one after the other; one call instead of two keeps
+ * the host's share of a decode step small. */
+int mlk_fused_moe(const void *w1, const void *w2, const void *x, const void *logits, int n_tokens,
+                  int n_router_experts, int n_experts, int topk, int hidden, int inter, int w_kind, int x_kind,
+                  int score_fun, int n_groups, int topk_groups, const void *bias, int renormalize,
+                  const int32_t *experts_map, const float *w1_scale, const float *w2_scale, int32_t *topk_ids,
+                  void *topk_weights, void *y, void *workspace, size_t workspace_bytes, void *stream);
+
 /* How mlk_fused_experts_compute would run one pass of min(n_tokens, 256) tokens; the launch code reads the same
  * plan.  out[0] = kernel family (0 single-token GeMV kernels, 1 decode kernels that align in-kernel, 2 decode
  * kernels after the alignment kernel, 3 row-shared kernels, 4 panel kernels: soft-FP8 weights with more than 64

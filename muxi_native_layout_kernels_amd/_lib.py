@@ -42,6 +42,9 @@ SIGNATURES = {
     "mlk_fused_experts_compute": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int,
                                           c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p,
                                           c_void_p, c_size_t, c_void_p]),
+    "mlk_fused_moe": (c_int, [c_void_p, c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                              c_int, c_int, c_int, c_int, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p,
+                              c_void_p, c_void_p, c_void_p, c_size_t, c_void_p]),
     "mlk_moe_workspace_bytes": (c_size_t, [c_int, c_int, c_int, c_int, c_int]),
     "mlk_moe_plan": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_void_p]),
 }

@@ -91,23 +91,32 @@ __device__ __forceinline__ uint32_t wave_argmax(const float (&v)[NE], int lane) 
     return ~wave_max_u32(~(bk == top ? bi : 0xffffffffu));   // lowest index among the holders
 }
 
-// One wave per token.  Expert lane + 64 i lives in register slot i of its lane.
-template <class T>
-__global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__ logits, int n_tokens, int E,
-                                                    int n_groups, int topk_groups, int topk, int score_fun,
-                                                    const uint16_t *__restrict__ bias, int renorm,
-                                                    int32_t *__restrict__ ids, uint16_t *__restrict__ weights) {
-    __shared__ __align__(16) double ex[kMaxExperts];   // exp(x - max), for the index-order sum
-    __shared__ __align__(16) float sel[kMaxExperts];   // selection scores, for the group scores
-    __shared__ int keep[kMaxExperts];
-    __shared__ int pick_id[kMaxTopK];
-    __shared__ float pick_w[kMaxTopK];
-    constexpr int NE = kMaxExperts / 64;
-    constexpr float kLowest = -3.0e38f;
+// LDS of one routing wave.
+struct RouterLds {
+    __align__(16) double ex[kMaxExperts];   // exp(x - max), for the index-order sum
+    __align__(16) float sel[kMaxExperts];   // selection scores, for the group scores
+    int keep[kMaxExperts];
+    int pick_id[kMaxTopK];
+    float pick_w[kMaxTopK];
+};
 
-    const int tok = blockIdx.x;
-    const int lane = threadIdx.x;
-    const uint16_t *row = logits + (size_t)tok * E;
+// The lanes of one wave exchange values through LDS: the LDS unit runs a wave's accesses in program order, so
+// all that is needed between a store and the loads of other lanes is that the compiler keeps that order.  (A
+// workgroup barrier would do too, but this code also runs in a single wave of a larger workgroup.)
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// Routing of one token by one wave; experts lane + 64 i live in register slot i of their lane (NE slots, so up
+// to 64 NE experts).  On return lane a < topk holds pick a (id and weight bits, in output order; the weight is
+// renormalised if asked for).
+template <class T, int NE>
+__device__ __forceinline__ void route_token(const uint16_t *__restrict__ row, int E, int n_groups, int topk_groups,
+                                            int topk, int score_fun, const uint16_t *__restrict__ bias, int renorm,
+                                            RouterLds &L, int lane, int &out_id, uint16_t &out_w) {
+    constexpr float kLowest = -3.0e38f;
     auto round_T = [](float v) { return T::to_f32(T::from_f32(v)); };
 
     // scores: exp, the index-order sum and the division in float64, one rounding to fp32, one to T
@@ -129,14 +138,14 @@ __global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__
         // LDS and come back sixteen at a time (eight 16-byte reads in flight), then add in order.
 #pragma unroll
         for (int i = 0; i < NE; ++i)
-            if (lane + 64 * i < E) ex[lane + 64 * i] = ev[i];
-        __syncthreads();
+            if (lane + 64 * i < E) L.ex[lane + 64 * i] = ev[i];
+        wave_lds_sync();
         typedef __attribute__((ext_vector_type(2))) double f64x2;
         double s = 0.0;
         for (int j0 = 0; j0 < E; j0 += 16) {
             f64x2 r[8];
 #pragma unroll
-            for (int t = 0; t < 8; ++t) r[t] = *reinterpret_cast<const f64x2 *>(&ex[j0 + 2 * t]);
+            for (int t = 0; t < 8; ++t) r[t] = *reinterpret_cast<const f64x2 *>(&L.ex[j0 + 2 * t]);
 #pragma unroll
             for (int t = 0; t < 8; ++t) {
                 if (j0 + 2 * t < E) s += r[t][0];
@@ -160,8 +169,8 @@ __global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__
         // group scores: max of the group, or the T-sum of its two largest positive scores with a bias
 #pragma unroll
         for (int i = 0; i < NE; ++i)
-            if (lane + 64 * i < E) sel[lane + 64 * i] = sv[i];
-        __syncthreads();
+            if (lane + 64 * i < E) L.sel[lane + 64 * i] = sv[i];
+        wave_lds_sync();
         const int per_group = E / n_groups;
         float gs[NE];
         int kept[NE];
@@ -171,7 +180,7 @@ __global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__
             gs[i] = kLowest;
             kept[i] = 0;
             if (g < n_groups) {
-                const float *seg = sel + g * per_group;
+                const float *seg = L.sel + g * per_group;
                 float score = 0.f;
                 if (!bias) {
 #pragma unroll 8
@@ -201,12 +210,12 @@ __global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__
         }
 #pragma unroll
         for (int i = 0; i < NE; ++i)
-            if (lane + 64 * i < n_groups) keep[lane + 64 * i] = kept[i];
-        __syncthreads();
+            if (lane + 64 * i < n_groups) L.keep[lane + 64 * i] = kept[i];
+        wave_lds_sync();
 #pragma unroll
         for (int i = 0; i < NE; ++i) {
             const int j = lane + 64 * i;
-            if (j < E && !keep[j / per_group]) { sv[i] = 0.f; pv[i] = 0.f; }
+            if (j < E && !L.keep[j / per_group]) { sv[i] = 0.f; pv[i] = 0.f; }
         }
     }
 
@@ -214,32 +223,32 @@ __global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__
     for (int kk = 0; kk < topk; ++kk) {
         const uint32_t pick = wave_argmax<NE>(sv, lane);
         if ((int)(pick & 63u) == lane) {
-            pick_id[kk] = (int)pick;
+            L.pick_id[kk] = (int)pick;
 #pragma unroll
             for (int i = 0; i < NE; ++i)
-                if (i == (int)(pick >> 6)) { pick_w[kk] = pv[i]; sv[i] = 0.f; }
+                if (i == (int)(pick >> 6)) { L.pick_w[kk] = pv[i]; sv[i] = 0.f; }
         }
     }
-    __syncthreads();
+    wave_lds_sync();
 
     // Lane a now takes pick a.  The softmax variant returns its picks ordered by expert id (stable for
     // equal ids): each lane counts the picks that go before its own and moves its pick there.
-    int my_id = lane < topk ? pick_id[lane] : 0x7fffffff;
-    float my_w = lane < topk ? pick_w[lane] : 0.f;
+    int my_id = lane < topk ? L.pick_id[lane] : 0x7fffffff;
+    float my_w = lane < topk ? L.pick_w[lane] : 0.f;
     if (score_fun == 0) {
         int before = 0;
         for (int b = 0; b < topk; ++b) {
             const int ib = __builtin_amdgcn_readlane(my_id, b);
             before += (ib < my_id || (ib == my_id && b < lane)) ? 1 : 0;
         }
-        __syncthreads();
+        wave_lds_sync();
         if (lane < topk) {
-            pick_id[before] = my_id;
-            pick_w[before] = my_w;
+            L.pick_id[before] = my_id;
+            L.pick_w[before] = my_w;
         }
-        __syncthreads();
-        my_id = lane < topk ? pick_id[lane] : 0x7fffffff;
-        my_w = lane < topk ? pick_w[lane] : 0.f;
+        wave_lds_sync();
+        my_id = lane < topk ? L.pick_id[lane] : 0x7fffffff;
+        my_w = lane < topk ? L.pick_w[lane] : 0.f;
     }
     float denom = 1.f;
     if (renorm) {
@@ -247,10 +256,26 @@ __global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__
         for (int a = 0; a < topk; ++a) s += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_w), a));
         denom = round_T(s);
     }
+    out_id = my_id;
+    out_w = (uint16_t)T::from_f32(renorm ? my_w / denom : my_w);
+}
+
+// One wave per token.
+template <class T>
+__global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__ logits, int n_tokens, int E,
+                                                    int n_groups, int topk_groups, int topk, int score_fun,
+                                                    const uint16_t *__restrict__ bias, int renorm,
+                                                    int32_t *__restrict__ ids, uint16_t *__restrict__ weights) {
+    __shared__ RouterLds L;
+    const int tok = blockIdx.x;
+    const int lane = threadIdx.x;
+    int id;
+    uint16_t w;
+    route_token<T, kMaxExperts / 64>(logits + (size_t)tok * E, E, n_groups, topk_groups, topk, score_fun, bias, renorm,
+                                     L, lane, id, w);
     if (lane < topk) {
-        ids[(size_t)tok * topk + lane] = my_id;
-        const float w = renorm ? my_w / denom : my_w;
-        weights[(size_t)tok * topk + lane] = (uint16_t)T::from_f32(w);
+        ids[(size_t)tok * topk + lane] = id;
+        weights[(size_t)tok * topk + lane] = w;
     }
 }
 
@@ -905,11 +930,11 @@ template <class T, bool FP8, int U>
 __global__ void __launch_bounds__(1024) moe_gate_up_gemv1_kernel(Moe1Args p) {
     extern __shared__ u32x4 xs[];          // the token's hidden vector
     __shared__ float red[16][16];
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int e = p.topk_ids[blockIdx.y];
     if (p.experts_map) e = p.experts_map[e];
     if (e < 0 || e >= p.E) return;
-    const int lane = threadIdx.x & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int stream = wave / (p.G * p.WK);
     const int gl = (wave / p.WK) % p.G, ks = wave % p.WK;
     constexpr int WB = FP8 ? 1 : 2;
@@ -1449,11 +1474,11 @@ extern "C" size_t mlk_moe_workspace_bytes(int n_tokens, int n_experts, int topk,
     return bytes;
 }
 
-extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const void *x, int n_tokens, int n_experts,
-                                         int topk, int hidden, int inter, int w_kind, int x_kind,
-                                         const int32_t *topk_ids, const void *topk_weights,
-                                         const int32_t *experts_map, const float *w1_scale, const float *w2_scale,
-                                         void *y, void *workspace, size_t workspace_bytes, void *stream) {
+static int experts_compute_impl(const void *w1, const void *w2, const void *x, int n_tokens, int n_experts,
+                                int topk, int hidden, int inter, int w_kind, int x_kind,
+                                const int32_t *topk_ids, const void *topk_weights,
+                                const int32_t *experts_map, const float *w1_scale, const float *w2_scale,
+                                void *y, void *workspace, size_t workspace_bytes, void *stream) {
     MLK_REQUIRE(x_kind == MLK_F16 || x_kind == MLK_BF16, "moe: activations must be fp16 or bf16");
     MLK_REQUIRE(n_tokens >= 0, "moe: negative token count");
     MLK_REQUIRE(n_experts >= 1 && n_experts <= kMaxExperts, "moe: 1..256 experts");
@@ -1580,4 +1605,36 @@ extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const v
         if (rc != MLK_OK) return rc;
     }
     return MLK_OK;
+}
+
+extern "C" int mlk_fused_experts_compute(const void *w1, const void *w2, const void *x, int n_tokens, int n_experts,
+                                         int topk, int hidden, int inter, int w_kind, int x_kind,
+                                         const int32_t *topk_ids, const void *topk_weights,
+                                         const int32_t *experts_map, const float *w1_scale, const float *w2_scale,
+                                         void *y, void *workspace, size_t workspace_bytes, void *stream) {
+    return experts_compute_impl(w1, w2, x, n_tokens, n_experts, topk, hidden, inter, w_kind, x_kind, topk_ids,
+                                topk_weights, experts_map, w1_scale, w2_scale, y, workspace, workspace_bytes, stream);
+}
+
+extern "C" int mlk_fused_moe(const void *w1, const void *w2, const void *x, const void *logits, int n_tokens,
+                             int n_router_experts, int n_experts, int topk, int hidden, int inter, int w_kind,
+                             int x_kind, int score_fun, int n_groups, int topk_groups, const void *bias,
+                             int renormalize, const int32_t *experts_map, const float *w1_scale,
+                             const float *w2_scale, int32_t *topk_ids, void *topk_weights, void *y, void *workspace,
+                             size_t workspace_bytes, void *stream) {
+    // the router's own argument checks, whoever routes
+    MLK_REQUIRE(x_kind == MLK_F16 || x_kind == MLK_BF16, "router: logits must be fp16 or bf16");
+    MLK_REQUIRE(score_fun == 0 || score_fun == 1, "router: score function must be 0 (softmax) or 1 (sigmoid)");
+    MLK_REQUIRE(n_tokens >= 0, "router: negative token count");
+    MLK_REQUIRE(n_router_experts >= 1 && n_router_experts <= kMaxExperts, "router: 1..256 experts");
+    MLK_REQUIRE(n_groups >= 1 && n_router_experts % n_groups == 0, "router: n_groups must divide the expert count");
+    MLK_REQUIRE(topk_groups >= 1 && topk_groups <= n_groups, "router: topk_groups must be in 1..n_groups");
+    MLK_REQUIRE(topk >= 1 && topk <= kMaxTopK && topk <= n_router_experts, "router: topk must be in 1..min(32, experts)");
+    if (n_tokens == 0) return MLK_OK;
+    MLK_REQUIRE(logits && topk_ids && topk_weights, "router: null pointer");
+    const int rc = mlk_fused_routing_gate(logits, x_kind, score_fun, n_tokens, n_router_experts, n_groups, topk_groups,
+                                          topk, bias, renormalize, topk_ids, topk_weights, stream);
+    if (rc != MLK_OK) return rc;
+    return experts_compute_impl(w1, w2, x, n_tokens, n_experts, topk, hidden, inter, w_kind, x_kind, topk_ids,
+                                topk_weights, experts_map, w1_scale, w2_scale, y, workspace, workspace_bytes, stream);
 }

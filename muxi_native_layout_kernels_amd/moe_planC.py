@@ -1,9 +1,9 @@
 """Fused MoE layer entry point; same signature and defaults as the reference's
 `muxi_moe_planC.fused_moe` (muxi_layout_kernels/muxi_moe_planC.py:6-149).
 
-Three library calls per layer: router (scores, grouped selection, top-K and the
-optional renormalisation in one kernel), then alignment + grouped gate/up GeMM +
-grouped down GeMM inside `mlk_fused_experts_compute`.  Apart from the output
+One library call per layer (`mlk_fused_moe`): router (scores, grouped selection,
+top-K and the optional renormalisation), alignment, grouped gate/up GeMM and
+grouped down GeMM.  Apart from the output
 nothing is allocated after the first call of a given shape: routing tables and
 the kernel workspace are cached per device and stream and are never freed, so a
 HIP graph captured around this function stays valid whatever runs later.
@@ -78,9 +78,18 @@ def fused_moe(
     ops._check(hidden_states.is_cuda and hidden_states.is_contiguous(), "hidden_states must be a contiguous CUDA tensor")
     ops._check(hidden_states.dtype in ops._KIND, "hidden_states must be fp16 or bf16")
     ops._check(gating_output.dtype == hidden_states.dtype, "gating_output must have the activation dtype")
+    # the router's argument checks (ops.fused_routing_gate), done here because one library call runs the whole layer
+    n_router_experts = gating_output.size(-1)
+    ops._check(gating_output.is_cuda and gating_output.is_contiguous(), "gating_output must be a contiguous CUDA tensor")
+    ops._check(B * n_router_experts == gating_output.numel(), "batch_size does not match gating_output")
+    ops._check(1 <= n_router_experts <= 256, "the router supports at most 256 experts")
+    ops._check(num_expert_group >= 1 and n_router_experts % num_expert_group == 0,
+               "n_groups must divide the number of experts")
+    ops._check(1 <= topk_group <= num_expert_group, "topK_groups must be in 1..n_groups")
+    ops._check(1 <= topk <= min(32, n_router_experts), "topK must be in 1..min(32, experts)")
+    if gating_bias is not None:
+        ops._check(gating_bias.dtype == gating_output.dtype, "Mismatched dtypes: load_balance_bias and gating_output.")
     topk_ids, topk_weights = _routing_buffers(B, topk, hidden_states.dtype, hidden_states.device)
-    ops.fused_routing_gate(gating_output, score_fun, B, H, num_expert_group, topk_group, topk_ids, topk_weights, topk,
-                           gating_bias, renormalize=bool(renormalize))
 
     if w1.dim() == 5:
         e1, m1, k1 = w1.shape[0], w1.shape[1] * 16, w1.shape[2] * 8
@@ -116,6 +125,6 @@ def fused_moe(
         experts_map = experts_map.to(torch.int)
 
     y = torch.empty_like(hidden_states)
-    ops.experts_compute_raw(w1, w2, hidden_states, B, e1, topk, H, k2, w_kind, topk_ids, topk_weights, experts_map,
-                            w1_scale, w2_scale, y)
+    ops.fused_moe_raw(w1, w2, hidden_states, gating_output, B, e1, topk, H, k2, w_kind, score_fun, num_expert_group,
+                      topk_group, gating_bias, renormalize, experts_map, w1_scale, w2_scale, topk_ids, topk_weights, y)
     return y.view(shape)

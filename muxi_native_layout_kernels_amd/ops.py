@@ -577,6 +577,19 @@ def experts_compute_raw(w1, w2, x, T, E, K, hidden, inter, w_kind, topk_ids, top
                                              _stream()), "fused_experts_compute")
 
 
+def fused_moe_raw(w1, w2, x, logits, T, E, K, hidden, inter, w_kind, score_fun, n_groups, topk_groups, bias,
+                  renormalize, experts_map, w1_scale, w2_scale, topk_ids, topk_weights, y):
+    """Thin call of the whole-layer entry point (router + alignment + both grouped GeMMs + weighted sum); no
+    checks.  `topk_ids` / `topk_weights` receive the routing."""
+    lib = _lib.load()
+    ws = _moe_workspace(x.device, lib.mlk_moe_workspace_bytes(T, E, K, hidden, inter))
+    _lib.check(lib.mlk_fused_moe(_ptr(w1), _ptr(w2), _ptr(x), _ptr(logits), T, logits.size(-1), E, K, hidden, inter,
+                                 w_kind, _KIND[x.dtype], score_fun, n_groups, topk_groups, _ptr(bias),
+                                 int(bool(renormalize)), _ptr(experts_map), _ptr(w1_scale), _ptr(w2_scale),
+                                 _ptr(topk_ids), _ptr(topk_weights), _ptr(y), _ptr(ws), ws.numel(), _stream()),
+               "fused_moe")
+
+
 # ------------------------------------------------- names outside the hot path
 def _out_of_scope(name, why):
     def fn(*args, **kwargs):
@@ -602,4 +615,5 @@ __all__ = [
     "routing_gate", "experts_compute", "fused_routing_gate",
     "batched_routed_activation_indexed_to_expert_block_indexed", "fused_experts_compute",
     "pack_layout_a", "unpack_layout_a", "experts_compute_raw", "release_workspaces", "workspace_bytes_held",
+    "fused_moe_raw",
 ]

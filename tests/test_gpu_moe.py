@@ -272,6 +272,30 @@ def test_fused_moe_single_token(mlk, dtype, fp8, E, K, H, I):
     assert_close(y1, y2.double().cpu().numpy(), RTOL, ATOL, "single-token kernels vs grouped kernels")
 
 
+@pytest.mark.parametrize("dtype,fp8,T,E,K,score,groups,with_bias", [
+    (torch.bfloat16, False, 1, 8, 2, "softmax", None, False),       # the Mixtral routing
+    (torch.float16, False, 1, 8, 2, "softmax", None, False),
+    (torch.bfloat16, True, 7, 8, 2, "softmax", None, False),
+    (torch.bfloat16, False, 33, 64, 8, "sigmoid", (8, 4), True),
+    (torch.bfloat16, True, 1, 48, 6, "softmax", (4, 2), False),     # expert count that is no power of two
+])
+def test_whole_layer_call_leaves_the_routing_in_its_buffers(mlk, dtype, fp8, T, E, K, score, groups, with_bias):
+    """`mlk_fused_moe` (one library call per layer) writes the router's picks into the ids / weights buffers it is
+    given: they must be the oracle's bit for bit, and the layer output must pass the same check as ever."""
+    from muxi_native_layout_kernels_amd import moe_planC
+    H, I = 256, 384
+    bias = randn((E,), dtype, 0.05, 55).abs() if with_bias else None
+    n_groups, tk_groups = groups if groups else (1, 1)
+    ids_buf, w_buf = moe_planC._routing_buffers(T, K, dtype, torch.device("cuda", torch.cuda.current_device()))
+    ids_buf.fill_(-7)
+    w_buf.zero_()
+    _moe_case(mlk, T, E, K, H, I, dtype, 4000 + T, score=score, fp8=fp8, groups=groups, bias=bias)
+    logits = randn((T, E), dtype, 1.0, 4000 + T + 1)
+    ids_o, w_o = orouter.route(logits, 0 if score == "softmax" else 1, n_groups, tk_groups, K, bias)
+    assert torch.equal(ids_buf.cpu(), ids_o)
+    assert torch.equal(w_buf.cpu().view(torch.int16), orouter.renormalize(w_o).view(torch.int16))
+
+
 @pytest.mark.parametrize("slices", [2, 4])
 @pytest.mark.parametrize("T,E,K,fp8", [(3, 8, 2, False), (16, 16, 8, False), (9, 8, 2, True)])
 def test_fused_moe_decode_k_sliced_down(mlk, slices, T, E, K, fp8):
