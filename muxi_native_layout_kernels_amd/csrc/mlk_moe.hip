@@ -260,8 +260,8 @@ __device__ __forceinline__ void route_token(const uint16_t *__restrict__ row, in
     out_w = (uint16_t)T::from_f32(renorm ? my_w / denom : my_w);
 }
 
-// One wave per token.
-template <class T>
+// One wave per token; NE register slots per lane hold up to 64 NE experts.
+template <class T, int NE>
 __global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__ logits, int n_tokens, int E,
                                                     int n_groups, int topk_groups, int topk, int score_fun,
                                                     const uint16_t *__restrict__ bias, int renorm,
@@ -271,8 +271,7 @@ __global__ void __launch_bounds__(64) router_kernel(const uint16_t *__restrict__
     const int lane = threadIdx.x;
     int id;
     uint16_t w;
-    route_token<T, kMaxExperts / 64>(logits + (size_t)tok * E, E, n_groups, topk_groups, topk, score_fun, bias, renorm,
-                                     L, lane, id, w);
+    route_token<T, NE>(logits + (size_t)tok * E, E, n_groups, topk_groups, topk, score_fun, bias, renorm, L, lane, id, w);
     if (lane < topk) {
         ids[(size_t)tok * topk + lane] = id;
         weights[(size_t)tok * topk + lane] = w;
@@ -923,6 +922,7 @@ struct Moe1Args {
     int K, H, I, E;
     int G, WK;                // gate/up: row groups per workgroup and waves splitting K (2*G*WK waves)
     int DW;                   // down: waves per workgroup
+    int prefetch;             // gate/up: bytes of every (pick, output row group) of W2 that the last workgroups touch ahead
 };
 
 // gate/up for one token: grid (I/(16 G), K); waves = (gate, up) x G row groups x WK slices of K
@@ -962,6 +962,30 @@ __global__ void __launch_bounds__(1024) moe_gate_up_gemv1_kernel(Moe1Args p) {
         }
         const float h = g / (1.f + __expf(-g)) * u;
         p.Hd[(size_t)blockIdx.y * p.I + (blockIdx.x * p.G + g_local) * 16 + r] = (uint16_t)T::from_f32(h);
+    }
+    // The grid's last workgroups run while the chip drains (fewer workgroups than slots are left) and the memory
+    // system has room: each of them reads the head of one output row group of the down projection, for every pick,
+    // so that the down kernel finds the first bytes it asks for in the Infinity Cache instead of in HBM.  The
+    // values are thrown away.
+    if (p.prefetch > 0) {
+        const int total = gridDim.x * gridDim.y, groups_h = p.H >> 4;
+        const int t = blockIdx.y * gridDim.x + blockIdx.x - (total - groups_h);
+        if (t >= 0) {
+            const size_t rg_bytes = (size_t)p.I * 16 * WB;
+            const size_t pf = (size_t)p.prefetch < rg_bytes ? (size_t)p.prefetch : rg_bytes;
+            u32x4 sink = {0u, 0u, 0u, 0u};
+            for (int k = 0; k < p.K; ++k) {
+                int e2 = p.topk_ids[k];
+                if (p.experts_map) e2 = p.experts_map[e2];
+                if (e2 < 0 || e2 >= p.E) continue;
+                const uint8_t *src = p.W2 + (size_t)e2 * p.H * p.I * WB + (size_t)t * rg_bytes;
+                for (size_t off = (size_t)threadIdx.x * 16; off + 16 <= pf; off += (size_t)blockDim.x * 16) {
+                    const u32x4 v = ld_global_u32x4(src + off);
+                    sink[0] ^= v[0] ^ v[1] ^ v[2] ^ v[3];
+                }
+            }
+            asm volatile("" ::"v"(sink[0]));
+        }
     }
 }
 
@@ -1433,14 +1457,23 @@ extern "C" int mlk_fused_routing_gate(const void *logits, int x_kind, int score_
     if (n_tokens == 0) return MLK_OK;
     MLK_REQUIRE(logits && ids && weights, "router: null pointer");
     hipStream_t s = (hipStream_t)stream;
-    if (x_kind == MLK_F16)
-        router_kernel<F16><<<n_tokens, 64, 0, s>>>((const uint16_t *)logits, n_tokens, n_experts, n_groups,
-                                                   topk_groups, topk, score_fun, (const uint16_t *)bias, renormalize,
-                                                   ids, (uint16_t *)weights);
-    else
-        router_kernel<BF16><<<n_tokens, 64, 0, s>>>((const uint16_t *)logits, n_tokens, n_experts, n_groups,
-                                                    topk_groups, topk, score_fun, (const uint16_t *)bias,
-                                                    renormalize, ids, (uint16_t *)weights);
+    // one, two or four experts per lane: a small expert count does not pay for the register slots of a large one
+#define MLK_ROUTER(TT, NE)                                                                                       \
+    router_kernel<TT, NE><<<n_tokens, 64, 0, s>>>((const uint16_t *)logits, n_tokens, n_experts, n_groups,       \
+                                                  topk_groups, topk, score_fun, (const uint16_t *)bias,          \
+                                                  renormalize, ids, (uint16_t *)weights)
+    // group counts above 64 also live in the register slots
+    const int widest = n_experts > n_groups ? n_experts : n_groups;
+    if (x_kind == MLK_F16) {
+        if (widest <= 64) MLK_ROUTER(F16, 1);
+        else if (widest <= 128) MLK_ROUTER(F16, 2);
+        else MLK_ROUTER(F16, 4);
+    } else {
+        if (widest <= 64) MLK_ROUTER(BF16, 1);
+        else if (widest <= 128) MLK_ROUTER(BF16, 2);
+        else MLK_ROUTER(BF16, 4);
+    }
+#undef MLK_ROUTER
     MLK_LAUNCH_CHECK();
     return MLK_OK;
 }
@@ -1531,6 +1564,7 @@ static int experts_compute_impl(const void *w1, const void *w2, const void *x, i
             m.G = G;
             m.WK = WK;
             m.DW = DW;
+            m.prefetch = g_tunable[13] * 1024;
             const dim3 g1(inter / (16 * G), topk), g2(hidden / 16);
             const int b1 = 2 * G * WK * 64, b2 = DW * 64;
             const size_t l1 = (size_t)hidden * 2, l2 = (size_t)topk * inter * 2;

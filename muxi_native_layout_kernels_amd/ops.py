@@ -23,6 +23,23 @@ def _stream():
     return torch.cuda.current_stream().cuda_stream
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+
+
+def _stream_of(t):
+    """Raw handle of torch's current stream on the tensor's device (the short way when torch offers it)."""
+    if _raw_stream is not None:
+        return _raw_stream(t.get_device())
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+# Launch plans of the eager entry points.  The first call with a given combination of shapes, dtypes and device
+# runs every argument check and the table lookup, and leaves the launch arguments here; later calls with the same
+# combination only check what a shape does not tell (contiguity, alpha / beta), allocate the output and call the
+# library.  A plan is a few integers: the cache is never cleared.
+_plans = {}
+
+
 def _ptr(t):
     return 0 if t is None else t.data_ptr()
 
@@ -239,6 +256,34 @@ def gemv_layoutA_wapper(A, B, m, k, alpha=1, beta=0, blockDimX=256, kernelId=1, 
 
 def gemv_layoutA(A, B, alpha=1, beta=0, scale_matrix=None, bias=None):
     """y[1, m] = alpha * B[1, k] . A^T (+ bias), A in layout-A (csrc/gemv_layout_a.cu:73-150)."""
+    key = ("gemv", A.shape, B.shape, A.dtype, B.dtype, A.device, B.device,
+           None if scale_matrix is None else (scale_matrix.shape, scale_matrix.dtype, scale_matrix.device),
+           None if bias is None else (bias.shape, bias.dtype, bias.device))
+    plan = _plans.get(key)
+    if plan is not None and beta == 0 and A.is_contiguous() and B.is_contiguous() and \
+            (scale_matrix is None or scale_matrix.is_contiguous()) and (bias is None or bias.is_contiguous()):
+        m, k, a_kind, x_kind, block, kid, p1, p2, use_scale, fn = plan
+        C = torch.empty((1, m), dtype=B.dtype, device=B.device)
+        rc = fn(A.data_ptr(), B.data_ptr(), C.data_ptr(), 1, m, k, a_kind, x_kind, alpha,
+                0 if bias is None else bias.data_ptr(), scale_matrix.data_ptr() if use_scale else 0,
+                block, kid, p1, p2, _stream_of(B))
+        if rc != 0:
+            _lib.check(rc, "gemv_layoutA")
+        return C
+    C = _gemv_layoutA_checked(A, B, alpha, beta, scale_matrix, bias)
+    m, k = A.size(0) * 16, A.size(1) * 8
+    if _is_fp8(A) and B.dtype == torch.bfloat16:
+        table = "gemv_soft_fp8"
+    else:
+        table = "gemv_fp16" if B.dtype == torch.float16 else "gemv_bf16"
+    block, kid, p1, p2 = arg_selector.gemv_guard(arg_selector.selector(table).get_args((m, k)), m, k)
+    _plans[key] = (m, k, _kind(A), _KIND[B.dtype], block, kid, p1, p2, _is_fp8(A) and scale_matrix is not None,
+                   _lib.load().mlk_gemv_layout_a)
+    return C
+
+
+def _gemv_layoutA_checked(A, B, alpha=1, beta=0, scale_matrix=None, bias=None):
+    """Every argument check of the reference's host launcher, the table lookup, the launch."""
     _check(A.is_cuda, "A must be a CUDA tensor")
     _check(B.is_cuda, "B must be a CUDA tensor")
     _check(A.is_contiguous(), "A must be contiguous")
@@ -307,6 +352,39 @@ def _gemm_guard(args, m):
     return args
 
 
+def _gemm_eager(tag, table, checked, A, A_Scale, B, alpha, beta, bias, b_mode, c_mode):
+    """The table-driven GeMM entry points behind their launch plans (see `_plans`): `checked` is the function that
+    runs every argument check, the table lookup and the launch for a combination not seen before."""
+    key = (tag, A.shape, B.shape, A.dtype, B.dtype, A.device, B.device,
+           None if A_Scale is None else (A_Scale.shape, A_Scale.dtype, A_Scale.device),
+           None if bias is None else (bias.shape, bias.dtype, bias.device))
+    plan = _plans.get(key)
+    if plan is not None and beta == 0 and A.is_contiguous() and B.is_contiguous() and \
+            (A_Scale is None or A_Scale.is_contiguous()) and (bias is None or bias.is_contiguous()):
+        m, n, k, a_kind, x_kind, kid, p1, p2, p3, ws_need, counter_bytes, use_scale, c_shape, fn = plan
+        C = torch.empty(c_shape, dtype=B.dtype, device=B.device)
+        stream = _stream_of(B)
+        ws_ptr = ws_len = 0
+        if p3 > 1:
+            ws = _gemm_pool.get(B.device, stream, ws_need, counter_bytes)
+            ws_ptr, ws_len = ws.data_ptr(), ws.numel()
+        rc = fn(A.data_ptr(), B.data_ptr(), C.data_ptr(), n, m, k, a_kind, x_kind, b_mode, c_mode, alpha,
+                0 if bias is None else bias.data_ptr(), A_Scale.data_ptr() if use_scale else 0, kid, p1, p2, p3,
+                ws_ptr, ws_len, stream)
+        if rc != 0:
+            _lib.check(rc, tag)
+        return C
+    C = checked()
+    lib = _lib.load()
+    m, k = A.size(0) * 16, A.size(1) * 8
+    n = B.size(0) if b_mode == _B_ROWMAJOR else B.size(1) * 16
+    kid, p1, p2, p3 = _gemm_guard(arg_selector.selector(table).get_args((m, n, k)), m)
+    _plans[key] = (m, n, k, _kind(A), _KIND[B.dtype], kid, p1, p2, p3,
+                   lib.mlk_gemm_workspace_bytes(n, m, int(p1), int(p3)) if p3 > 1 else 0, lib.mlk_gemm_counter_bytes(),
+                   _is_fp8(A) and A_Scale is not None, tuple(C.shape), lib.mlk_gemm_layout_a)
+    return C
+
+
 def gemm_layoutA_wapper(A, B, m, n, k, alpha=1, beta=0, kernelParam1=1, kernelParam2=1, kernelParam3=1, kernelId=1,
                         bias=None):
     """csrc/gemm_layout_A.cu:684-750 with explicit launch parameters."""
@@ -324,6 +402,12 @@ def _check_gemm_common(A, B):
 def gemm_layoutA(A, B, alpha=1, beta=0, bias=None):
     """C[n, m] = alpha * B[n, k] . A^T (+ bias); A layout-A, B and C row-major
     (csrc/gemm_layout_A.cu:752-787)."""
+    return _gemm_eager("gemm_layoutA", "layoutA_gemm", lambda: _gemm_layoutA_checked(A, B, alpha, beta, bias), A, None, B, alpha, beta, bias,
+                       _B_ROWMAJOR, _C_ROWMAJOR)
+
+
+def _gemm_layoutA_checked(A, B, alpha=1, beta=0, bias=None):
+    """Every argument check of the reference's host launcher, the table lookup, the launch."""
     _check_gemm_common(A, B)
     m, a_k = _layout_a_dims(A)
     _check(B.dim() == 2, "B must be a 2D tensor")
@@ -347,6 +431,12 @@ def gemm_layoutA_soft_fp8_wapper(A, A_Scale, B, m, n, k, alpha=1, beta=0, kernel
 def gemm_layoutA_soft_fp8(A, A_Scale, B, alpha=1, beta=0, bias=None):
     """Soft-FP8 weights (e4m3 bytes in layout-A + fp32 scale per 128x128 block), bf16
     activations (csrc/gemm_layout_A_soft_fp8.cu:825-862)."""
+    return _gemm_eager("gemm_layoutA_soft_fp8", "layoutA_soft_fp8_gemm", lambda: _gemm_layoutA_soft_fp8_checked(A, A_Scale, B, alpha, beta, bias), A, A_Scale, B, alpha,
+                       beta, bias, _B_ROWMAJOR, _C_ROWMAJOR)
+
+
+def _gemm_layoutA_soft_fp8_checked(A, A_Scale, B, alpha=1, beta=0, bias=None):
+    """Every argument check of the reference's host launcher, the table lookup, the launch."""
     _check_gemm_common(A, B)
     m, a_k = _layout_a_dims(A)
     _check(B.dim() == 2, "B must be a 2D tensor")
@@ -384,6 +474,12 @@ def gemm_layoutAB_ContinuousC_wapper(A, B, m, n, k, alpha=1, beta=0, kernelParam
 
 def gemm_layoutAB_ContinuousC(A, B, alpha=1, beta=0, bias=None):
     """A layout-A, B layout-B, C row-major [n, m] (csrc/gemm_layout_ab_continuous_c.cu:1051-1093)."""
+    return _gemm_eager("gemm_layoutAB_ContinuousC", "continuous_gemm", lambda: _gemm_layoutAB_ContinuousC_checked(A, B, alpha, beta, bias), A, None, B, alpha, beta, bias,
+                       _B_NATIVE, _C_ROWMAJOR)
+
+
+def _gemm_layoutAB_ContinuousC_checked(A, B, alpha=1, beta=0, bias=None):
+    """Every argument check of the reference's host launcher, the table lookup, the launch."""
     _check_gemm_common(A, B)
     m, a_k = _layout_a_dims(A)
     n, b_k = _native_b_dims(B)
@@ -405,6 +501,12 @@ def gemm_layoutABC_wapper(A, B, m, n, k, alpha=1, beta=0, kernelParam1=1, kernel
 def gemm_layoutABC(A, B, alpha=1, beta=0, bias=None):
     """A layout-A, B layout-B, C layout-C [m/32, n/16, 4, 16, 8], ready to be the B of the
     next product (csrc/gemm_layout_abc.cu:754-791)."""
+    return _gemm_eager("gemm_layoutABC", "layout_gemm", lambda: _gemm_layoutABC_checked(A, B, alpha, beta, bias), A, None, B, alpha, beta, bias,
+                       _B_NATIVE, _C_NATIVE)
+
+
+def _gemm_layoutABC_checked(A, B, alpha=1, beta=0, bias=None):
+    """Every argument check of the reference's host launcher, the table lookup, the launch."""
     _check_gemm_common(A, B)
     m, a_k = _layout_a_dims(A)
     n, b_k = _native_b_dims(B)

@@ -441,3 +441,26 @@ def test_gemm_errors(mlk):
     with pytest.raises(RuntimeError, match="data type"):
         mlk.gemm_layoutA(a, b.half())
     assert mlk.gemm_layoutA(a, b).shape == (16, 128)
+
+
+def test_gemm_repeated_calls_take_the_launch_plan_and_keep_the_checks(mlk):
+    """Second calls with the same shapes run from the launch plan: same results as the first, K-split workspace
+    included, and the per-call checks (contiguity, beta) still raise."""
+    n, k, m = 1024, 2048, 24
+    w = randn((n, k), torch.float16, 0.02, 51)
+    a = pack_a(w).cuda()
+    b1, b2 = randn((m, k), torch.float16, 1.0, 52).cuda(), randn((m, k), torch.float16, 1.0, 53).cuda()
+    c1 = mlk.gemm_layoutA(a, b1)
+    c2 = mlk.gemm_layoutA(a, b2)                                  # planned
+    c1b = mlk.gemm_layoutA(a, b1)                                 # planned
+    assert torch.equal(c1, c1b)
+    assert_close(c2, ogemm.linear_expected(w, b2.cpu()), RTOL, ATOL, "planned call")
+    bn = mlk.layoutB(randn((32, k), torch.float16, 1.0, 54).cuda())
+    for fn in (mlk.gemm_layoutABC, mlk.gemm_layoutAB_ContinuousC):
+        assert torch.equal(fn(a, bn), fn(a, bn))
+    assert torch.equal(mlk.reLayoutC(mlk.gemm_layoutABC(a, bn)), mlk.gemm_layoutAB_ContinuousC(a, bn))
+    with pytest.raises(RuntimeError, match="beta"):
+        mlk.gemm_layoutA(a, b1, beta=2)
+    wide = torch.zeros((m, 2 * k), dtype=torch.float16, device="cuda")
+    with pytest.raises(RuntimeError, match="contiguous"):
+        mlk.gemm_layoutA(a, wide[:, ::2])

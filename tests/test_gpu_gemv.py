@@ -171,3 +171,26 @@ def test_gemv_matrix_core_variant_all_codes_exact(mlk):
                                         kernelParam2=2, scale_matrix=scale.cuda())
             want = softfp8.bf16_bits_to_f32(softfp8.dequant_bf16_bits(codes.numpy(), np.float32(s)))
             assert np.array_equal(y.cpu().float().numpy().reshape(-1), want)
+
+
+def test_gemv_repeated_calls_take_the_launch_plan_and_keep_the_checks(mlk):
+    """The second call with the same shapes and dtypes skips the shape checks and the table lookup (launch plan);
+    what a shape does not tell is still checked on every call, and other values of alpha / bias go through."""
+    n, k = 512, 1024
+    w = randn((n, k), torch.bfloat16, 0.05, 41)
+    a = pack_a(w).cuda()
+    x1, x2 = randn((1, k), torch.bfloat16, 1.0, 42).cuda(), randn((1, k), torch.bfloat16, 1.0, 43).cuda()
+    bias = randn((1, n), torch.bfloat16, 1.0, 44).cuda()
+    y1 = mlk.gemv_layoutA(a, x1)
+    y2 = mlk.gemv_layoutA(a, x2)                                  # planned
+    assert_close(y1, ogemm.linear_expected(w, x1.cpu()), RTOL, ATOL, "first call")
+    assert_close(y2, ogemm.linear_expected(w, x2.cpu()), RTOL, ATOL, "planned call")
+    y3 = mlk.gemv_layoutA(a, x2, alpha=0.5, bias=bias)
+    y4 = mlk.gemv_layoutA(a, x1, alpha=0.25, bias=bias)           # planned, other alpha
+    assert_close(y3, ogemm.linear_expected(w, x2.cpu(), 0.5, bias.cpu()), RTOL, ATOL, "bias, first call")
+    assert_close(y4, ogemm.linear_expected(w, x1.cpu(), 0.25, bias.cpu()), RTOL, ATOL, "bias, planned call")
+    with pytest.raises(RuntimeError, match="beta"):
+        mlk.gemv_layoutA(a, x1, beta=1)
+    wide = torch.zeros((1, 2 * k), dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(RuntimeError, match="contiguous"):
+        mlk.gemv_layoutA(a, wide[:, ::2])                         # same shape and dtype, not contiguous
