@@ -922,7 +922,6 @@ struct Moe1Args {
     int K, H, I, E;
     int G, WK;                // gate/up: row groups per workgroup and waves splitting K (2*G*WK waves)
     int DW;                   // down: waves per workgroup
-    int prefetch;             // gate/up: bytes of every (pick, output row group) of W2 that the last workgroups touch ahead
 };
 
 // gate/up for one token: grid (I/(16 G), K); waves = (gate, up) x G row groups x WK slices of K
@@ -962,30 +961,6 @@ __global__ void __launch_bounds__(1024) moe_gate_up_gemv1_kernel(Moe1Args p) {
         }
         const float h = g / (1.f + __expf(-g)) * u;
         p.Hd[(size_t)blockIdx.y * p.I + (blockIdx.x * p.G + g_local) * 16 + r] = (uint16_t)T::from_f32(h);
-    }
-    // The grid's last workgroups run while the chip drains (fewer workgroups than slots are left) and the memory
-    // system has room: each of them reads the head of one output row group of the down projection, for every pick,
-    // so that the down kernel finds the first bytes it asks for in the Infinity Cache instead of in HBM.  The
-    // values are thrown away.
-    if (p.prefetch > 0) {
-        const int total = gridDim.x * gridDim.y, groups_h = p.H >> 4;
-        const int t = blockIdx.y * gridDim.x + blockIdx.x - (total - groups_h);
-        if (t >= 0) {
-            const size_t rg_bytes = (size_t)p.I * 16 * WB;
-            const size_t pf = (size_t)p.prefetch < rg_bytes ? (size_t)p.prefetch : rg_bytes;
-            u32x4 sink = {0u, 0u, 0u, 0u};
-            for (int k = 0; k < p.K; ++k) {
-                int e2 = p.topk_ids[k];
-                if (p.experts_map) e2 = p.experts_map[e2];
-                if (e2 < 0 || e2 >= p.E) continue;
-                const uint8_t *src = p.W2 + (size_t)e2 * p.H * p.I * WB + (size_t)t * rg_bytes;
-                for (size_t off = (size_t)threadIdx.x * 16; off + 16 <= pf; off += (size_t)blockDim.x * 16) {
-                    const u32x4 v = ld_global_u32x4(src + off);
-                    sink[0] ^= v[0] ^ v[1] ^ v[2] ^ v[3];
-                }
-            }
-            asm volatile("" ::"v"(sink[0]));
-        }
     }
 }
 
@@ -1193,7 +1168,8 @@ static size_t carve(uint8_t *base, int tc, int E, int K, int hidden, int inter, 
     const int n_pairs = tc * K;
     const int max_padded = n_pairs + E * 15;
     int max_blocks = (max_padded + 15) / 16;
-    if (max_blocks < kDecodePairs) max_blocks = kDecodePairs;   // the in-kernel alignment numbers blocks by task
+    // the in-kernel alignment numbers blocks by task: at most one block per routed pair, kDecodePairs at most
+    if (max_blocks < (n_pairs < kDecodePairs ? n_pairs : kDecodePairs)) max_blocks = n_pairs < kDecodePairs ? n_pairs : kDecodePairs;
     size_t off = 0;
     auto take = [&](size_t bytes) {
         uint8_t *ptr = base ? base + off : nullptr;
@@ -1537,7 +1513,7 @@ static int experts_compute_impl(const void *w1, const void *w2, const void *x, i
         carve((uint8_t *)workspace, tc, n_experts, topk, hidden, inter, &ws);
         const int max_padded = n_pairs + n_experts * 15;
         int max_blocks = (max_padded + 15) / 16;
-        if (max_blocks < kDecodePairs) max_blocks = kDecodePairs;
+        if (max_blocks < (n_pairs < kDecodePairs ? n_pairs : kDecodePairs)) max_blocks = n_pairs < kDecodePairs ? n_pairs : kDecodePairs;
         const int max_tasks = pl.max_tasks;
         // one token: every routed pair is a GeMV with the activations in LDS
         if (pl.path == kMoePathGemv1) {
@@ -1564,7 +1540,6 @@ static int experts_compute_impl(const void *w1, const void *w2, const void *x, i
             m.G = G;
             m.WK = WK;
             m.DW = DW;
-            m.prefetch = g_tunable[13] * 1024;
             const dim3 g1(inter / (16 * G), topk), g2(hidden / 16);
             const int b1 = 2 * G * WK * 64, b2 = DW * 64;
             const size_t l1 = (size_t)hidden * 2, l2 = (size_t)topk * inter * 2;

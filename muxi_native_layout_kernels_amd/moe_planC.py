@@ -17,6 +17,7 @@ from . import ops
 
 _cache_lock = threading.Lock()
 _route_cache = {}
+_plans = {}
 
 
 def _routing_buffers(n_tokens, topk, dtype, device, stream=None):
@@ -59,6 +60,29 @@ def fused_moe(
     experts_map: Optional[torch.Tensor] = None,
 ) -> torch.Tensor:
     """The MetaX tile parameters (APerWarp .. block_dim_x_gemm) are accepted and ignored."""
+    # A combination of shapes, dtypes, devices and options that has passed every check below before runs from its
+    # launch plan: per call only contiguity is checked again (a shape does not tell it).
+    key = (hidden_states.shape, hidden_states.dtype, hidden_states.device, w1.shape, w1.dtype, w1.device, w2.shape,
+           w2.dtype, w2.device, gating_output.shape, gating_output.dtype, gating_output.device, topk, bool(renormalize),
+           use_grouped_topk, num_expert_group, topk_group, score_func, soft_fp8,
+           None if w1_scale is None else (w1_scale.shape, w1_scale.dtype, w1_scale.device),
+           None if w2_scale is None else (w2_scale.shape, w2_scale.dtype, w2_scale.device),
+           None if block_shape is None else tuple(block_shape),
+           None if gating_bias is None else (gating_bias.shape, gating_bias.dtype, gating_bias.device),
+           None if experts_map is None else (experts_map.shape, experts_map.dtype, experts_map.device))
+    plan = _plans.get(key)
+    if plan is not None and hidden_states.is_contiguous() and w1.is_contiguous() and w2.is_contiguous() and \
+            gating_output.is_contiguous() and (w1_scale is None or w1_scale.is_contiguous()) and \
+            (w2_scale is None or w2_scale.is_contiguous()) and (gating_bias is None or gating_bias.is_contiguous()) and \
+            (experts_map is None or experts_map.is_contiguous()):
+        B, H, E, I, w_kind, score_fun, n_groups, k_groups, scaled = plan
+        topk_ids, topk_weights = _routing_buffers(B, topk, hidden_states.dtype, hidden_states.device,
+                                                  ops._stream_of(hidden_states))
+        y = torch.empty_like(hidden_states)
+        ops.fused_moe_raw(w1, w2, hidden_states, gating_output, B, E, topk, H, I, w_kind, score_fun, n_groups, k_groups,
+                          gating_bias, renormalize, experts_map, w1_scale if scaled else None,
+                          w2_scale if scaled else None, topk_ids, topk_weights, y)
+        return y
     assert hidden_states.shape[0] == gating_output.shape[0], "Number of tokens mismatch"
     if num_expert_group is None:
         num_expert_group = 1
@@ -127,4 +151,6 @@ def fused_moe(
     y = torch.empty_like(hidden_states)
     ops.fused_moe_raw(w1, w2, hidden_states, gating_output, B, e1, topk, H, k2, w_kind, score_fun, num_expert_group,
                       topk_group, gating_bias, renormalize, experts_map, w1_scale, w2_scale, topk_ids, topk_weights, y)
+    if experts_map is None or experts_map.dtype == torch.int:      # (a converted map is a new tensor every call)
+        _plans[key] = (B, H, e1, k2, w_kind, score_fun, num_expert_group, topk_group, w1_scale is not None)
     return y.view(shape)
