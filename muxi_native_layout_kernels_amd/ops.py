@@ -264,7 +264,7 @@ def gemv_layoutA(A, B, alpha=1, beta=0, scale_matrix=None, bias=None):
             (scale_matrix is None or scale_matrix.is_contiguous()) and (bias is None or bias.is_contiguous()):
         m, k, a_kind, x_kind, block, kid, p1, p2, use_scale, fn = plan
         C = torch.empty((1, m), dtype=B.dtype, device=B.device)
-        rc = fn(A.data_ptr(), B.data_ptr(), C.data_ptr(), 1, m, k, a_kind, x_kind, alpha,
+        rc = fn(A.data_ptr(), B.data_ptr(), C.data_ptr(), 1, m, k, a_kind, x_kind, float(alpha),
                 0 if bias is None else bias.data_ptr(), scale_matrix.data_ptr() if use_scale else 0,
                 block, kid, p1, p2, _stream_of(B))
         if rc != 0:
@@ -368,7 +368,7 @@ def _gemm_eager(tag, table, checked, A, A_Scale, B, alpha, beta, bias, b_mode, c
         if p3 > 1:
             ws = _gemm_pool.get(B.device, stream, ws_need, counter_bytes)
             ws_ptr, ws_len = ws.data_ptr(), ws.numel()
-        rc = fn(A.data_ptr(), B.data_ptr(), C.data_ptr(), n, m, k, a_kind, x_kind, b_mode, c_mode, alpha,
+        rc = fn(A.data_ptr(), B.data_ptr(), C.data_ptr(), n, m, k, a_kind, x_kind, b_mode, c_mode, float(alpha),
                 0 if bias is None else bias.data_ptr(), A_Scale.data_ptr() if use_scale else 0, kid, p1, p2, p3,
                 ws_ptr, ws_len, stream)
         if rc != 0:
