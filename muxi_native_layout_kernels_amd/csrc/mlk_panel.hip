@@ -43,8 +43,105 @@ struct PanelArgs {
     int SK;              // K slices of the row tiles from whole_groups * 8 on
     int whole_groups;    // groups of eight row tiles in front that are not sliced (0: every row tile has SK slices)
     int row_tiles, token_tiles;
+    int band, chunk;     // gemm_panel8_kernel: groups of row tiles and token tiles that neighbouring workgroups of an XCD cover
     float alpha;
 };
+
+// What happens to the accumulators of a panel: scaled and stored, or (K slices) handed over as fp32 partials that the
+// last workgroup to arrive adds in slice order.  acc[pr][tb] covers the row groups rg0 + 2 pr, + 1 and the 32 tokens from
+// tok0 + 32 tb on; NWAVES waves per workgroup, each with PR x TB accumulators; the fold fetches FB accumulators at a time.
+template <class T, int PR, int TB, int NWAVES, int FB>
+__device__ __forceinline__ void panel_finish(const PanelArgs &p, f32x16 (&acc)[PR][TB], int rg0, int tok0, int SK, int sk,
+                                             int rt, int tt, int wave, int lane, int *s_last) {
+    const int groups = p.N >> 4;
+    // accumulator element 4 g + e of lane 32 h + c: weight row 8 g + 4 h + e of the pair's 32, token c of the block's 32
+    const int half = lane >> 5, c32 = lane & 31;
+    auto epilogue = [&](int pr, int tb, int g, f32x4 v) {
+        const int n = (rg0 + 2 * pr) * 16 + 8 * g + 4 * half;
+        const int tok = tok0 + tb * 32 + c32;
+        if ((n >> 4) >= groups || tok >= p.M) return;
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            o[i] = p.alpha * v[i];
+            if (p.bias) o[i] += T::to_f32(p.bias[n + i]);
+        }
+        store4<T>(p.C + (size_t)tok * p.N + n, o[0], o[1], o[2], o[3]);
+    };
+    auto quad = [&](const f32x16 &v, int g) { return f32x4{v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3]}; };
+    if (SK == 1) {
+#pragma unroll
+        for (int pr = 0; pr < PR; ++pr)
+#pragma unroll
+            for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+                for (int g = 0; g < 4; ++g) epilogue(pr, tb, g, quad(acc[pr][tb], g));
+        return;
+    }
+    const int tile = (rt - p.whole_groups * 8) * p.token_tiles + tt;               // among the sliced tiles
+    const int tiles = (p.row_tiles - p.whole_groups * 8) * p.token_tiles;
+    // 64-lane group of quad jj of this wave in slice s (two planes of 8-byte halves, see st_agent_planar)
+    auto group_at = [&](int s, int jj) -> f32x4 * {
+        return p.partial + ((((size_t)s * tiles + tile) * NWAVES + wave) * (PR * TB * 4) + jj) * 64;
+    };
+    // partials travel as agent-scope (write-through / always-miss) accesses, like in the narrow kernels; a release /
+    // acquire fence pair around ordinary stores was measured slower (it writes back and invalidates a whole L2)
+#pragma unroll
+    for (int pr = 0; pr < PR; ++pr)
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) st_agent_planar(group_at(sk, (pr * TB + tb) * 4 + g), 64, lane, quad(acc[pr][tb], g));
+    __builtin_amdgcn_s_waitcnt(0);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int prev = __hip_atomic_fetch_add(&p.counters[tile], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *s_last = (prev == SK - 1);
+        if (*s_last) __hip_atomic_store(&p.counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    __syncthreads();
+    if (!*s_last) return;
+    // slice order; the loads of the next slice are in flight while the current one is added (a round trip to
+    // memory per slice would otherwise be paid in full: these loads bypass the caches).  FB accumulators are fetched
+    // at a time: all of a row pair's where the registers allow it.
+    static_assert(TB % FB == 0, "fetch groups are whole accumulators of one row pair");
+#pragma unroll
+    for (int pr = 0; pr < PR; ++pr) {
+#pragma unroll
+        for (int t0b = 0; t0b < TB; t0b += FB) {
+#pragma unroll
+            for (int tb = 0; tb < FB; ++tb)
+#pragma unroll
+                for (int e = 0; e < 16; ++e) acc[pr][t0b + tb][e] = 0.f;
+            f32x4 t0[FB * 4], t1[FB * 4];
+            auto fetch = [&](f32x4 (&t)[FB * 4], int sl) {
+#pragma unroll
+                for (int jj = 0; jj < FB * 4; ++jj) t[jj] = ld_agent_planar(group_at(sl, (pr * TB + t0b) * 4 + jj), 64, lane);
+            };
+            auto add = [&](const f32x4 (&t)[FB * 4]) {
+#pragma unroll
+                for (int tb = 0; tb < FB; ++tb)
+#pragma unroll
+                    for (int e = 0; e < 16; ++e) acc[pr][t0b + tb][e] += t[tb * 4 + (e >> 2)][e & 3];
+            };
+            fetch(t0, 0);
+            for (int sl = 0; sl < SK; sl += 2) {
+                if (sl + 1 < SK) fetch(t1, sl + 1);
+                add(t0);
+                if (sl + 1 < SK) {
+                    if (sl + 2 < SK) fetch(t0, sl + 2);
+                    add(t1);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int pr = 0; pr < PR; ++pr)
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+            for (int g = 0; g < 4; ++g) epilogue(pr, tb, g, quad(acc[pr][tb], g));
+}
 
 template <class T, bool FP8, int TB, int PR>
 __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
@@ -109,98 +206,194 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     for (int pr = 0; pr < PR; ++pr) srows[pr] = srow;          // the row groups of a wave lie in one 128-row block
     PanelLoop<T, FP8, TB, PR>::run(acc, abase, srows, p.B, boff, wbeg, nwin, win);
 
-    // accumulator element 4 g + e of lane 32 h + c: weight row 8 g + 4 h + e of the pair's 32, token c of the block's 32
-    const int half = lane >> 5, c32 = lane & 31;
-    auto epilogue = [&](int pr, int tb, int g, f32x4 v) {
-        const int n = (rg0 + 2 * pr) * 16 + 8 * g + 4 * half;
-        const int tok = tok0 + tb * 32 + c32;
-        if ((n >> 4) >= groups || tok >= p.M) return;
-        float o[4];
+    panel_finish<T, PR, TB, kTileWaves, TB>(p, acc, rg0, tok0, SK, sk, rt, tt, wave, lane, &s_last);
+}
+
+// ---------------------------------------------------------------------------------------------------------------
+// 256 x 256 panels of 16-bit weights: eight waves, both operands through LDS, fetched with loads that write LDS directly.
+//
+// A wave that issues v_mfma_f32_32x32x16 back to back loses matrix-core time with every other instruction it has to
+// issue in between (measured: about 20 cycles per LDS read, 24 per load); with two waves per SIMD the instructions
+// of one wave go out under the products of the other.  That needs both waves of a SIMD inside 256 registers each,
+// so nothing is staged through registers here: a k32 slab of the panel (16 weight tiles of 16 rows x 32 k, 1 KiB
+// each, as they lie in layout A; 16 chunks of 16 tokens x 32 k) is copied into LDS by 32 buffer loads with the LDS
+// bit, four per wave: the weight tiles addressed by the thread id alone (the descriptor adds 16 bytes per lane, no
+// address register), the token chunks with a per-lane offset (lane 4 t + j fetches octet j ^ (t / 4) of token t, so that
+// four lanes cover 64 consecutive bytes of a token row and the operand reads below meet no bank twice).
+// Wave w = (token half w / 4, row quarter w % 4) multiplies 64 rows x 128 tokens: per k16 step two weight operands (two
+// vertically adjacent tiles read as one 32-row operand: lane 32 g + i takes row i % 16 of tile i / 16, octet g) and four
+// token operands feed eight products.
+//
+// Ring of four slabs (128 KiB).  While slab s is multiplied, slab s + 1 is complete and published, slab s + 2 is landing
+// and the loads of slab s + 3 go out into the buffer that slab s - 1 has left; one wait (this wave's loads of slab
+// s + 2) and one barrier per slab publish slab s + 2 and retire slab s.  The operands of the first step of slab s + 1
+// are read before that barrier, so no wave stands idle behind it.  The barrier is the bare instruction: the fence that
+// comes with __syncthreads() would wait for every load in flight.
+constexpr int kP8Slab = 2048;                                  // 16-byte granules of a slab: 1024 of weights, 1024 of tokens
+constexpr size_t kP8LdsBytes = (size_t)4 * kP8Slab * 16;
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt_le() {
+    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x70 | 0xF00);
+}
+__device__ __forceinline__ void bare_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// the four loads of one wave for slab `slab` (counted from k = 0) into ring buffer `buf`
+__device__ __forceinline__ void p8_issue(const uint8_t *a_panel, const uint16_t *b, const uint32_t (&a_soff)[2],
+                                         const uint32_t (&b_voff)[2], int wave, int slab, int buf) {
+    extern __shared__ u32x4 win[];
+    __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc((void *)a_panel, 16, 0xffffffffu, 1 << 23);
+    __amdgpu_buffer_rsrc_t rs_b = __builtin_amdgcn_make_buffer_rsrc((void *)b, 0, 0xffffffffu, 0x00020000);
+    const int dst = buf * kP8Slab;
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            o[i] = p.alpha * v[i];
-            if (p.bias) o[i] += T::to_f32(p.bias[n + i]);
-        }
-        store4<T>(p.C + (size_t)tok * p.N + n, o[0], o[1], o[2], o[3]);
-    };
-    auto quad = [&](const f32x16 &v, int g) { return f32x4{v[4 * g], v[4 * g + 1], v[4 * g + 2], v[4 * g + 3]}; };
-    if (SK == 1) {
+    for (int i = 0; i < 2; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, win + dst + (2 * wave + i) * 64, 16, 0, a_soff[i] + slab * 1024, 0, 0);
 #pragma unroll
-        for (int pr = 0; pr < PR; ++pr)
-#pragma unroll
-            for (int tb = 0; tb < TB; ++tb)
-#pragma unroll
-                for (int g = 0; g < 4; ++g) epilogue(pr, tb, g, quad(acc[pr][tb], g));
-        return;
+    for (int i = 0; i < 2; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, win + dst + 1024 + (2 * wave + i) * 64, 16, b_voff[i], slab * 64, 0, 0);
+}
+
+//
+// Grid: without K slices the workgroup ids of an XCD walk bands of p.band groups of eight row tiles in chunks of
+// p.chunk token tiles, so that the 32 workgroups an XCD runs at a time cover 8 x 4 (row tiles x token tiles) and share
+// both operands through its L2; with the token tiles of two row tiles side by side (2 x 16) the same product took
+// 17 % longer (8192 x 8192, 4096 tokens: 491 against 413 us).  A fifth slab of LDS (160 KiB) changed nothing.
+template <class T>
+__global__ void __launch_bounds__(512) gemm_panel8_kernel(PanelArgs p) {
+    constexpr int RING = 4;
+    extern __shared__ u32x4 win[];
+    constexpr int PR = 2, TB = 4;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wr = wave & 3, wt = wave >> 2;
+
+    // workgroup -> (row tile, k slice, token tile), as in gemm_panel_kernel
+    const int xcd = blockIdx.x & 7;
+    int u = blockIdx.x >> 3;
+    int SK, sk, tt, rt;
+    if (p.band > 0) {
+        const int TT = p.token_tiles, groups8 = (p.row_tiles + 7) >> 3, RB = p.band, TC = p.chunk;
+        const int band = u / (RB * TT);
+        const int nb = min(RB, groups8 - band * RB);           // groups of row tiles in this band
+        const int v = u - band * RB * TT;
+        const int c = v / (nb * TC);
+        const int tc = min(TC, TT - c * TC);                   // token tiles in this chunk
+        const int w = v - c * nb * TC;
+        SK = 1, sk = 0;
+        tt = c * TC + w % tc;
+        rt = (band * RB + w / tc) * 8 + xcd;
+    } else {
+        const int whole_wgs = p.whole_groups * p.token_tiles;
+        const bool sliced = u >= whole_wgs;
+        SK = sliced ? p.SK : 1;
+        if (sliced) u -= whole_wgs;
+        tt = u % p.token_tiles;
+        u /= p.token_tiles;
+        sk = u % SK;
+        rt = ((sliced ? p.whole_groups : 0) + u / SK) * 8 + xcd;
     }
-    const int tile = (rt - p.whole_groups * 8) * p.token_tiles + tt;               // among the sliced tiles
-    const int tiles = (p.row_tiles - p.whole_groups * 8) * p.token_tiles;
-    // 64-lane group of quad jj of this wave in slice s (two planes of 8-byte halves, see st_agent_planar)
-    auto group_at = [&](int s, int jj) -> f32x4 * {
-        return p.partial + ((((size_t)s * tiles + tile) * kTileWaves + wave) * (PR * TB * 4) + jj) * 64;
-    };
-    // partials travel as agent-scope (write-through / always-miss) accesses, like in the narrow kernels; a release /
-    // acquire fence pair around ordinary stores was measured slower (it writes back and invalidates a whole L2)
+    if (rt >= p.row_tiles) return;
+
+    const int groups = p.N >> 4;
+    const int rgp = rt * 16;                                   // first row group of the panel
+    const int rg0 = rgp + wr * 4;                              // of this wave
+    const int tok0 = tt * 256;
+    const int nwin_total = p.K / 64;                           // slices are cut in windows of 64 k, as the host counts them
+    const int wbeg = (int)((long long)sk * nwin_total / SK);
+    const int slab0 = 2 * wbeg;
+    const int nslab = 2 * ((int)((long long)(sk + 1) * nwin_total / SK) - wbeg);
+
+    // sources of this wave's loads: weight tiles 2 wave, 2 wave + 1 of the panel (rows past N: a copy of the last row
+    // group, never stored), token chunks 2 wave, 2 wave + 1 (tokens past M: the last token)
+    const uint8_t *a_panel = p.A + (size_t)rgp * p.K * 32;
+    uint32_t a_soff[2], b_voff[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int rg = min(rgp + 2 * wave + i, groups - 1);
+        a_soff[i] = (uint32_t)(rg - rgp) * (uint32_t)p.K * 32u;
+        const int t = lane >> 2, oct = (lane & 3) ^ ((t >> 2) & 3);
+        const int tok = min(tok0 + (2 * wave + i) * 16 + t, p.M - 1);
+        b_voff[i] = (uint32_t)tok * (uint32_t)p.K * 2u + oct * 16;
+    }
+    // operand reads (granules inside a slab, first k16 step; the second step is + 32 for weights, ^ 2 for tokens)
+    const int g = lane >> 5, i32 = lane & 31, t16 = i32 & 15, hi = i32 >> 4;
+    const int a_idx = (wr * 4 + hi) * 64 + g * 16 + t16;                                         // + 128 pr
+    const int b_idx = 1024 + (wt * 8 + hi) * 64 + 4 * t16 + (g ^ ((t16 >> 2) & 3));           // + 128 tb
+
+    f32x16 acc[PR][TB];
 #pragma unroll
     for (int pr = 0; pr < PR; ++pr)
-#pragma unroll
-        for (int tb = 0; tb < TB; ++tb)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) st_agent_planar(group_at(sk, (pr * TB + tb) * 4 + g), 64, lane, quad(acc[pr][tb], g));
-    __builtin_amdgcn_s_waitcnt(0);
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int prev = __hip_atomic_fetch_add(&p.counters[tile], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (prev == SK - 1);
-        if (s_last) __hip_atomic_store(&p.counters[tile], 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
-    __syncthreads();
-    if (!s_last) return;
-    // slice order; the loads of the next slice are in flight while the current one is added (a round trip to
-    // memory per slice would otherwise be paid in full: these loads bypass the caches)
-#pragma unroll
-    for (int pr = 0; pr < PR; ++pr) {
 #pragma unroll
         for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[pr][tb][e] = 0.f;
-        f32x4 t0[TB * 4], t1[TB * 4];
-        auto fetch = [&](f32x4 (&t)[TB * 4], int sl) {
+
+    u32x4 a0[PR], a1[PR], b0[TB], b1[TB];
+    auto rd = [&](u32x4 (&a)[PR], u32x4 (&b)[TB], int buf, int hs) {
+        const u32x4 *src = win + buf * kP8Slab;
 #pragma unroll
-            for (int jj = 0; jj < TB * 4; ++jj) t[jj] = ld_agent_planar(group_at(sl, pr * TB * 4 + jj), 64, lane);
-        };
-        auto add = [&](const f32x4 (&t)[TB * 4]) {
+        for (int pr = 0; pr < PR; ++pr) a[pr] = src[a_idx + 128 * pr + hs * 32];
 #pragma unroll
-            for (int tb = 0; tb < TB; ++tb)
-#pragma unroll
-                for (int e = 0; e < 16; ++e) acc[pr][tb][e] += t[tb * 4 + (e >> 2)][e & 3];
-        };
-        fetch(t0, 0);
-        for (int sl = 0; sl < SK; sl += 2) {
-            if (sl + 1 < SK) fetch(t1, sl + 1);
-            add(t0);
-            if (sl + 1 < SK) {
-                if (sl + 2 < SK) fetch(t0, sl + 2);
-                add(t1);
-            }
-        }
-    }
-#pragma unroll
-    for (int pr = 0; pr < PR; ++pr)
+        for (int tb = 0; tb < TB; ++tb) b[tb] = src[(b_idx ^ (hs * 2)) + 128 * tb];
+    };
+    auto mm = [&](const u32x4 (&a)[PR], const u32x4 (&b)[TB]) {
 #pragma unroll
         for (int tb = 0; tb < TB; ++tb)
 #pragma unroll
-            for (int g = 0; g < 4; ++g) epilogue(pr, tb, g, quad(acc[pr][tb], g));
+            for (int pr = 0; pr < PR; ++pr) acc[pr][tb] = T::mfma32(a[pr], b[tb], acc[pr][tb]);
+    };
+    // slabs past the end of the slice are fetched as copies of its last slab and never multiplied, which keeps the
+    // count of loads in flight the same in every trip
+    const int last = slab0 + nslab - 1;
+#pragma unroll
+    for (int i = 0; i < RING - 1; ++i) p8_issue(a_panel, p.B, a_soff, b_voff, wave, min(slab0 + i, last), i);
+    wait_vmcnt_le<4 * (RING - 3)>();                           // slabs 0 and 1 of this wave have landed
+    bare_barrier();
+    rd(a0, b0, 0, 0);
+    int cur = 0;                                               // ring buffer of slab s
+    for (int s = 0; s < nslab; ++s) {
+        const int nxt = cur == RING - 1 ? 0 : cur + 1, prv = cur == 0 ? RING - 1 : cur - 1;
+        p8_issue(a_panel, p.B, a_soff, b_voff, wave, min(slab0 + s + RING - 1, last), prv);
+        rd(a1, b1, cur, 1);
+        mm(a0, b0);
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (m != 3 && m != 7) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+            if (m < 4) __builtin_amdgcn_sched_group_barrier(0x020, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        rd(a0, b0, nxt, 0);
+        mm(a1, b1);
+#pragma unroll
+        for (int m = 0; m < 8; ++m) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+            if (m != 3 && m != 7) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        wait_vmcnt_le<4 * (RING - 3)>();                       // this wave's loads of slab s + 2 have landed
+        bare_barrier();
+        cur = nxt;
+    }
+    __builtin_amdgcn_s_waitcnt(0);                             // nothing may still be writing LDS when the ring is given up
+    mfma_settle();
+    __syncthreads();
+    panel_finish<T, PR, TB, 8, 2>(p, acc, rg0, tok0 + wt * 128, SK, sk, rt, tt, wave, lane, reinterpret_cast<int *>(win));
 }
 
-// Tokens per panel when the caller leaves the choice open.  Workgroups run one per CU in rounds, and a 256-token
-// panel takes 1.84 times as long as a 128-token one (measured), so the width with the cheaper sum of rounds wins.
-int panel_tokens(int m, int n) {
+// Tokens per panel when the caller leaves the choice open.  Workgroups run one per CU in rounds; a 256-token panel
+// takes 1.3 to 1.5 times as long as a 128-token one for 16-bit weights (eight-wave kernel) and 1.84 times for soft-FP8
+// ones (measured), so the width with the cheaper sum of rounds wins.
+int panel_tokens(int m, int n, bool fp8) {
     const int cus = device_cus();
     const long long row_tiles = (n + kPanelRowsPerWg - 1) / kPanelRowsPerWg;
     const long long rounds128 = (row_tiles * ((m + 127) / 128) + cus - 1) / cus;
     const long long rounds256 = (row_tiles * ((m + 255) / 256) + cus - 1) / cus;
-    return rounds256 * 184 < rounds128 * 100 ? 256 : 128;
+    return rounds256 * (fp8 ? 184 : 140) < rounds128 * 100 ? 256 : 128;
 }
 
 size_t panel_partial_bytes(int m, int n, int sk) {
@@ -228,7 +421,7 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
     p.N = n;
     p.K = k;
     p.alpha = alpha;
-    if (width != 128 && width != 256) width = panel_tokens(m, n);
+    if (width != 128 && width != 256) width = panel_tokens(m, n, a_kind == MLK_FP8_E4M3);
     p.token_tiles = (m + width - 1) / width;
     MLK_REQUIRE(k % 128 == 0, "gemm: the panel kernel needs K % 128 == 0");
     MLK_REQUIRE((long long)m * k < (1ll << 31), "gemm: the panel kernel indexes activations with 32 bits");
@@ -280,10 +473,28 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
         }                                                                                                          \
         gemm_panel_kernel<TT, F8, TBB, PRR><<<grid, 256, lds, s>>>(p);                                                  \
     } while (0)
-    if (width == 256) {
-        if (a_kind == MLK_FP8_E4M3) MLK_PANEL(BF16, true, 8, 2);
-        else if (a_kind == MLK_F16) MLK_PANEL(F16, false, 8, 2);
-        else MLK_PANEL(BF16, false, 8, 2);
+    if (width == 256 && a_kind != MLK_FP8_E4M3) {
+        // eight waves, operands through LDS
+#define MLK_PANEL8(TT)                                                                                                 \
+    do {                                                                                                           \
+        static bool ready_on[64] = {};                                                                             \
+        bool &ready = ready_on[dev & 63];                                                                          \
+        if (!ready) {                                                                                              \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_panel8_kernel<TT>),            \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kP8LdsBytes);     \
+            if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));                                \
+            ready = true;                                                                                          \
+        }                                                                                                          \
+        gemm_panel8_kernel<TT><<<grid, 512, kP8LdsBytes, s>>>(p);                                                  \
+    } while (0)
+        const bool whole = p.SK == 1 && p.whole_groups == 0;
+        p.band = whole ? 8 : 0;
+        p.chunk = 4;
+        if (a_kind == MLK_F16) MLK_PANEL8(F16);
+        else MLK_PANEL8(BF16);
+#undef MLK_PANEL8
+    } else if (width == 256) {
+        MLK_PANEL(BF16, true, 8, 2);
     } else if (rows == 256) {
         if (a_kind == MLK_FP8_E4M3) MLK_PANEL(BF16, true, 4, 2);
         else if (a_kind == MLK_F16) MLK_PANEL(F16, false, 4, 2);
