@@ -23,17 +23,22 @@
 #pragma once
 
 #include "mlk_moe_args.cuh"
-#include "mlk_panel_loop.cuh"
+#include "mlk_panel_lds.cuh"
 
 namespace mlk {
 
+// Slabs of LDS per workgroup.  Gate/up: four (56 or 64 KiB), two workgroups per CU.  Down: six (84 or 96 KiB), one
+// workgroup per CU: its grid is about one workgroup per CU, and two of them on one CU while another CU idles cost
+// more than the second wave per SIMD brings (Mixtral shape, 256 tokens: 179 against 137 us).
+constexpr int kMoeGateUpRing = 4, kMoeDownRing = 6;
+
 template <class T, bool FP8, int TB>
-__global__ void __launch_bounds__(256, 1) moe_gate_up_panel_kernel(MoeArgs p) {
+__global__ void __launch_bounds__(256, 2) moe_gate_up_panel_kernel(MoeArgs p) {
     extern __shared__ u32x4 win[];
     const int task = blockIdx.y;
     if (task >= p.n_tasks[0]) return;
     const MoeTask tk = p.tasks[task];
-    using Loop = PanelLoop<T, FP8, TB, 2>;
+    using Loop = PanelLoopLds<T, FP8, TB, kMoeGateUpRing>;
     constexpr int WB = FP8 ? 1 : 2;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -54,16 +59,12 @@ __global__ void __launch_bounds__(256, 1) moe_gate_up_panel_kernel(MoeArgs p) {
                                         scale_cols, lane);
     }
     const int slots = tk.nblocks * 16;
-    const int colg = tid % Loop::GPR, trow = tid / Loop::GPR;
-    uint32_t boff[Loop::NG];
-#pragma unroll
-    for (int i = 0; i < Loop::NG; ++i) {
-        const int slot = trow + Loop::RP * i;
+    auto row_off = [&](int slot) -> uint32_t {                 // the token row that slot `slot` of the task reads
         int id = p.n_pairs;
         if (slot < slots) id = p.sorted[tk.block0 * 16 + slot];
         const int tok = id < p.n_pairs ? id / p.K : 0;
-        boff[i] = (uint32_t)tok * (uint32_t)p.H + colg * 8;
-    }
+        return (uint32_t)tok * (uint32_t)p.H;
+    };
     f32x16 acc[2][TB];
 #pragma unroll
     for (int pr = 0; pr < 2; ++pr)
@@ -72,7 +73,7 @@ __global__ void __launch_bounds__(256, 1) moe_gate_up_panel_kernel(MoeArgs p) {
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[pr][tb][e] = 0.f;
 
-    Loop::run(acc, abase, srow, p.X, boff, 0, p.H >> 7, win);
+    Loop::run(acc, abase, srow, p.X, row_off, 0, p.H >> 5, win);
 
     // accumulator element 4 g + e of lane 32 h + c: row 8 g + 4 h + e of the pair's 32, token c of the block's 32
     const int half = lane >> 5, c32 = lane & 31;
@@ -96,12 +97,12 @@ __global__ void __launch_bounds__(256, 1) moe_gate_up_panel_kernel(MoeArgs p) {
 }
 
 template <class T, bool FP8, int TB>
-__global__ void __launch_bounds__(256, 1) moe_down_panel_kernel(MoeArgs p, float *__restrict__ O) {
+__global__ void __launch_bounds__(256, 2) moe_down_panel_kernel(MoeArgs p, float *__restrict__ O) {
     extern __shared__ u32x4 win[];
     const int task = blockIdx.y;
     if (task >= p.n_tasks[0]) return;
     const MoeTask tk = p.tasks[task];
-    using Loop = PanelLoop<T, FP8, TB, 2>;
+    using Loop = PanelLoopLds<T, FP8, TB, kMoeDownRing>;
     constexpr int WB = FP8 ? 1 : 2;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -118,14 +119,9 @@ __global__ void __launch_bounds__(256, 1) moe_down_panel_kernel(MoeArgs p, float
         srow[1] = srow[0];                                         // 64 rows from a multiple of 64: one 128-row block
     }
     const int slots = tk.nblocks * 16;
-    const int colg = tid % Loop::GPR, trow = tid / Loop::GPR;
-    uint32_t boff[Loop::NG];
-#pragma unroll
-    for (int i = 0; i < Loop::NG; ++i) {
-        int slot = trow + Loop::RP * i;
-        if (slot >= slots) slot = 0;
-        boff[i] = (uint32_t)(tk.block0 * 16 + slot) * (uint32_t)p.I + colg * 8;
-    }
+    auto row_off = [&](int slot) -> uint32_t {                 // rows of the intermediate, one per slot of the alignment
+        return (uint32_t)(tk.block0 * 16 + (slot < slots ? slot : 0)) * (uint32_t)p.I;
+    };
     f32x16 acc[2][TB];
 #pragma unroll
     for (int pr = 0; pr < 2; ++pr)
@@ -134,10 +130,10 @@ __global__ void __launch_bounds__(256, 1) moe_down_panel_kernel(MoeArgs p, float
 #pragma unroll
             for (int e = 0; e < 16; ++e) acc[pr][tb][e] = 0.f;
 
-    const int nwin_total = p.I >> 7;
+    const int nwin_total = p.I >> 7;                              // K slices are cut at multiples of 128 k
     const int wbeg = (int)((long long)blockIdx.z * nwin_total / (int)gridDim.z);
     const int nwin = (int)((long long)(blockIdx.z + 1) * nwin_total / (int)gridDim.z) - wbeg;
-    Loop::run(acc, abase, srow, p.Hbuf, boff, wbeg, nwin, win);
+    Loop::run(acc, abase, srow, p.Hbuf, row_off, 4 * wbeg, 4 * nwin, win);
 
     const int half = lane >> 5, c32 = lane & 31;
 #pragma unroll
@@ -175,15 +171,16 @@ static int panel_lds_attribute(K kernel, size_t lds, bool (&ready_on)[64]) {
 
 template <class T, bool FP8, int TB>
 static int launch_moe_panel_tb(const MoeArgs &a, int max_tasks, float *obuf, int skd, hipStream_t s) {
-    const size_t lds = panel_lds_bytes(TB);
+    const size_t lds = PanelLdsShape<FP8, TB, kMoeGateUpRing>::lds_bytes;
+    const size_t lds_down = PanelLdsShape<FP8, TB, kMoeDownRing>::lds_bytes;
     static bool ready_gate[64] = {}, ready_down[64] = {};
     int rc = panel_lds_attribute(&moe_gate_up_panel_kernel<T, FP8, TB>, lds, ready_gate);
     if (rc != MLK_OK) return rc;
-    rc = panel_lds_attribute(&moe_down_panel_kernel<T, FP8, TB>, lds, ready_down);
+    rc = panel_lds_attribute(&moe_down_panel_kernel<T, FP8, TB>, lds_down, ready_down);
     if (rc != MLK_OK) return rc;
     moe_gate_up_panel_kernel<T, FP8, TB><<<dim3(a.I / 128, max_tasks), 256, lds, s>>>(a);
     MLK_LAUNCH_CHECK();
-    moe_down_panel_kernel<T, FP8, TB><<<dim3(a.H / 256, max_tasks, skd), 256, lds, s>>>(a, obuf);
+    moe_down_panel_kernel<T, FP8, TB><<<dim3(a.H / 256, max_tasks, skd), 256, lds_down, s>>>(a, obuf);
     MLK_LAUNCH_CHECK();
     return MLK_OK;
 }
