@@ -401,13 +401,36 @@ def main():
             blas_yardstick(row, n, k, DT[kind], m, steps, count)
         return row
 
+    mfma_only = {}
+
+    def mfma_only_tflops(dt):
+        """Matrix-core yardstick: a loop of nothing but v_mfma_f32_32x32x16 on operand values drawn like the
+        benchmark's (weights 0.02 * N(0, 1), activations N(0, 1)), one workgroup of eight waves per CU, replayed
+        like the cases.  The power limit, not the instruction rate, sets what the chip sustains on such values."""
+        if dt not in mfma_only:
+            a = (torch.randn((64 * 1024,), generator=gen, device=dev) * 0.02).to(dt)
+            b = torch.randn((64 * 1024,), generator=gen, device=dev).to(dt)
+            cus = torch.cuda.get_device_properties(dev).multi_processor_count
+            iters = 4000
+
+            def call():
+                _lib.check(lib.mlk_mfma_probe(a.data_ptr(), b.data_ptr(), iters, cus, 0,
+                                              torch.cuda.current_stream().cuda_stream), "mfma_probe")
+            t = run_graph([call], 10, 3, reps=3, direct_if_short=True)
+            mfma_only[dt] = cus * 8 * iters * 16 * 32768.0 / t["us_median"] / 1e6
+        return mfma_only[dt]
+
     def panel_case(name, n, k, kind, m, steps):
         """Prefill-sized token counts: bound by the matrix cores (or by the weight stream up to ~300 tokens).
-        The vendor BLAS on an un-packed 16-bit copy of the same shape is timed beside it."""
+        The vendor BLAS on an un-packed 16-bit copy of the same shape is timed beside it, and the rate of a loop
+        that only issues the same MFMA instruction on like-valued operands (`mfma_only_tflops`)."""
         row = gemm_case(name, n, k, kind, m, steps, 3, copies=2, cpu=False)
         flops = 2.0 * m * n * k
         row["tflops"] = flops / row["us"] / 1e6
         row["mfma_frac"] = row["tflops"] / MFMA_PEAK_TFLOPS
+        if not args.counters:
+            row["mfma_only_tflops"] = mfma_only_tflops(torch.bfloat16)
+            row["frac_of_mfma_only"] = row["tflops"] / row["mfma_only_tflops"]
         row["bound"] = "mfma" if flops / (MFMA_PEAK_TFLOPS * 1e6) > row["bytes"] / (HBM_PEAK_GBPS * 1e3) else "hbm"
         dt = torch.bfloat16 if kind == 2 else DT[kind]
         W = [(torch.randn((n, k), generator=gen, device=dev) * 0.02).to(dt) for _ in range(2)]
@@ -715,7 +738,8 @@ def main():
             row.pop("wall", None)
             row.pop("how", None)
             for key in ("us", "us_first", "us_median", "us_min", "gbps", "frac", "roofline_us", "ratio_to_roofline", "tflops",
-                        "mfma_frac", "read_only_us", "blas_us", "blas_tflops", "traffic_over_algorithmic"):
+                        "mfma_frac", "read_only_us", "blas_us", "blas_tflops", "traffic_over_algorithmic",
+                        "mfma_only_tflops", "frac_of_mfma_only"):
                 if row.get(key) is not None:
                     row[key] = round(row[key], 4)
 

@@ -108,6 +108,13 @@ int mlk_fp8_weight_repack(const void *src, void *dst, int64_t nbytes, void *stre
  * system delivers to a pure streaming kernel next to the 8 TB/s peak.  No counterpart in the reference. */
 int mlk_stream_read(const void *src, int64_t nbytes, int block_dim_x, int workgroups, void *sink, void *stream);
 
+/* Measurement aid: `workgroups` workgroups of eight waves; every wave reads four 1 KiB operands from `a` and four from
+ * `b` (32 KiB each must be readable: 16-bit values, e.g. the head of a weight and of an activation matrix) and issues
+ * iters x 16 v_mfma_f32_32x32x16_bf16 on them, nothing else.  flops = workgroups x 8 x iters x 16 x 32768.  Used by
+ * bench.py to report the matrix-core rate the chip sustains on the benchmark's operand values (the power limit lowers
+ * the clock under dense random operands) next to the 2.5 PFLOP/s peak.  No counterpart in the reference. */
+int mlk_mfma_probe(const void *a, const void *b, int iters, int workgroups, void *sink, void *stream);
+
 /* ---------------------------------------------------------------------- GeMV
  * y[M, N] = T(alpha * x[M, K] . A^T (+ bias[N])), 1 <= M <= 4, fp32 accumulate,
  * A in layout-A.  Replaces `gemv_layoutA` / `gemv_layoutA_wapper`,

@@ -25,6 +25,7 @@ SIGNATURES = {
     "mlk_re_layout_c": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p]),
     "mlk_fp8_weight_repack": (c_int, [c_void_p, c_void_p, c_int64, c_void_p]),
     "mlk_stream_read": (c_int, [c_void_p, c_int64, c_int, c_int, c_void_p, c_void_p]),
+    "mlk_mfma_probe": (c_int, [c_void_p, c_void_p, c_int, c_int, c_void_p, c_void_p]),
     "mlk_gemv_layout_a": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_float,
                                   c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_void_p]),
     "mlk_gemm_layout_a": (c_int, [c_void_p, c_void_p, c_void_p, c_int, c_int, c_int, c_int, c_int, c_int, c_int,

@@ -30,10 +30,16 @@ namespace mlk {
 // Slabs of LDS per workgroup.  Gate/up: four (56 or 64 KiB), two workgroups per CU.  Down: six (84 or 96 KiB), one
 // workgroup per CU: its grid is about one workgroup per CU, and two of them on one CU while another CU idles cost
 // more than the second wave per SIMD brings (Mixtral shape, 256 tokens: 179 against 137 us).
-constexpr int kMoeGateUpRing = 4, kMoeDownRing = 6;
+#ifndef MLK_GU_RING
+#define MLK_GU_RING 4
+#endif
+#ifndef MLK_GU_OCC
+#define MLK_GU_OCC 2
+#endif
+constexpr int kMoeGateUpRing = MLK_GU_RING, kMoeDownRing = 6;
 
 template <class T, bool FP8, int TB>
-__global__ void __launch_bounds__(256, 2) moe_gate_up_panel_kernel(MoeArgs p) {
+__global__ void __launch_bounds__(256, MLK_GU_OCC) moe_gate_up_panel_kernel(MoeArgs p) {
     extern __shared__ u32x4 win[];
     const int task = blockIdx.y;
     if (task >= p.n_tasks[0]) return;

@@ -28,6 +28,7 @@
 // tiles by that XCD's L2.  K slices fold like in the row-shared kernel: fp32 partials with
 // agent-scope stores, the last workgroup to arrive adds them in slice order.
 #include "mlk_panel_loop.cuh"
+#include "mlk_panel_lds.cuh"
 
 namespace mlk {
 
@@ -209,6 +210,58 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
     panel_finish<T, PR, TB, kTileWaves, TB>(p, acc, rg0, tok0, SK, sk, rt, tt, wave, lane, &s_last);
 }
 
+// 256 x 128 panels on the loop of mlk_panel_lds.cuh (four waves, LDS as the prefetch buffer; soft-FP8: two workgroups
+// per CU).  Same grid and fold as gemm_panel_kernel.
+template <class T, bool FP8, int RING>
+__global__ void __launch_bounds__(256, 2) gemm_panel_lds_kernel(PanelArgs p) {
+    extern __shared__ u32x4 win[];
+    constexpr int TB = 4, PR = 2, R = 4;
+    constexpr int WBYTES = FP8 ? 1 : 2;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int xcd = blockIdx.x & 7;
+    int u = blockIdx.x >> 3;
+    const int whole_wgs = p.whole_groups * p.token_tiles;
+    const bool sliced = u >= whole_wgs;
+    const int SK = sliced ? p.SK : 1;
+    if (sliced) u -= whole_wgs;
+    const int tt = u % p.token_tiles;
+    u /= p.token_tiles;
+    const int sk = u % SK;
+    const int rt = ((sliced ? p.whole_groups : 0) + u / SK) * 8 + xcd;
+    if (rt >= p.row_tiles) return;
+
+    const int groups = p.N >> 4;
+    const int rg0 = (rt * kTileWaves + wave) * R;
+    const int tok0 = tt * (TB * 32);
+    const int nwin_total = p.K / 128;                          // slices are cut in windows of 128 k, as the host counts them
+    const int wbeg = (int)((long long)sk * nwin_total / SK);
+    const int nwin = (int)((long long)(sk + 1) * nwin_total / SK) - wbeg;
+    const int scale_cols = (p.K + 127) >> 7;
+    const uint8_t *abase[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const int rg = min(rg0 + r, groups - 1);              // rows past N are computed on a copy and never stored
+        abase[r] = p.A + (size_t)rg * p.K * 16 * WBYTES;
+    }
+    ScaleRow srows[PR];
+    if (FP8) {
+        srows[0] = load_scale_row(p.scale ? p.scale + (size_t)(min(rg0, groups - 1) >> 3) * scale_cols : nullptr, scale_cols, lane);
+        srows[1] = srows[0];                                   // the row groups of a wave lie in one 128-row block
+    }
+    auto row_off = [&](int slot) -> uint32_t { return (uint32_t)min(tok0 + slot, p.M - 1) * (uint32_t)p.K; };
+    f32x16 acc[PR][TB];
+#pragma unroll
+    for (int pr = 0; pr < PR; ++pr)
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[pr][tb][e] = 0.f;
+    PanelLoopLds<T, FP8, TB, RING>::run(acc, abase, srows, p.B, row_off, 4 * wbeg, 4 * nwin, win);
+    __syncthreads();                                           // the ring is given up: its first word takes the fold's flag
+    panel_finish<T, PR, TB, kTileWaves, 2>(p, acc, rg0, tok0, SK, sk, rt, tt, wave, lane, reinterpret_cast<int *>(win));
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // 256 x 256 panels of 16-bit weights: eight waves, both operands through LDS, fetched with loads that write LDS directly.
 //
@@ -231,16 +284,6 @@ __global__ void __launch_bounds__(256, 1) gemm_panel_kernel(PanelArgs p) {
 // comes with __syncthreads() would wait for every load in flight.
 constexpr int kP8Slab = 2048;                                  // 16-byte granules of a slab: 1024 of weights, 1024 of tokens
 constexpr size_t kP8LdsBytes = (size_t)4 * kP8Slab * 16;
-
-template <int N>
-__device__ __forceinline__ void wait_vmcnt_le() {
-    __builtin_amdgcn_s_waitcnt((N & 0xF) | ((N >> 4) << 14) | 0x70 | 0xF00);
-}
-__device__ __forceinline__ void bare_barrier() {
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
 
 // the four loads of one wave for slab `slab` (counted from k = 0) into ring buffer `buf`
 __device__ __forceinline__ void p8_issue(const uint8_t *a_panel, const uint16_t *b, const uint32_t (&a_soff)[2],
@@ -495,6 +538,25 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
 #undef MLK_PANEL8
     } else if (width == 256) {
         MLK_PANEL(BF16, true, 8, 2);
+    } else if (rows == 256 && a_kind == MLK_FP8_E4M3 && (p.SK == 1 || p.whole_groups > 0)) {
+        // soft-FP8, panels computed whole (or only the last round's sliced): the loop that prefetches through LDS, two
+        // workgroups per CU (28672 x 8192 at 1024 tokens: 616 -> 474 us); fully sliced grids and 16-bit weights stay on
+        // the register-ring loop, which is ahead there
+#define MLK_PANEL_LDS(TT, F8, RING)                                                                                    \
+    do {                                                                                                           \
+        constexpr size_t lds = PanelLdsShape<F8, 4, RING>::lds_bytes;                                              \
+        static bool ready_on[64] = {};                                                                             \
+        bool &ready = ready_on[dev & 63];                                                                          \
+        if (!ready) {                                                                                              \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_panel_lds_kernel<TT, F8, RING>), \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);             \
+            if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));                                \
+            ready = true;                                                                                          \
+        }                                                                                                          \
+        gemm_panel_lds_kernel<TT, F8, RING><<<grid, 256, lds, s>>>(p);                                             \
+    } while (0)
+        MLK_PANEL_LDS(BF16, true, 4);
+#undef MLK_PANEL_LDS
     } else if (rows == 256) {
         if (a_kind == MLK_FP8_E4M3) MLK_PANEL(BF16, true, 4, 2);
         else if (a_kind == MLK_F16) MLK_PANEL(F16, false, 4, 2);

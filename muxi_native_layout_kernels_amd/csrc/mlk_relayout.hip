@@ -129,6 +129,43 @@ __global__ void __launch_bounds__(256) fp8_repack16_kernel(const u32x4 *__restri
     }
 }
 
+// Matrix-core yardstick: every wave takes four 32-row operands from `a` and four from `b` (16 bytes per lane each, read
+// once) and issues iters x 16 v_mfma_f32_32x32x16_bf16 on them, eight waves per workgroup, nothing else in the loop and
+// nothing stored.  What it measures is the rate the chip sustains on those operand VALUES: with zeros the clock stays at
+// its maximum, with the dense random values of a real product the power limit pulls it down by a third.
+__global__ void __launch_bounds__(512) mfma_probe_kernel(const u32x4 *__restrict__ a, const u32x4 *__restrict__ b, int iters,
+                                                         uint32_t *__restrict__ sink) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    u32x4 x[4], y[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        x[i] = a[(wave * 4 + i) * 64 + lane];
+        y[i] = b[(wave * 4 + i) * 64 + lane];
+    }
+    f32x16 acc[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[i][j][e] = 0.f;
+    for (int it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int r = 0; r < 2; ++r)
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = BF16::mfma32(x[2 * r + i], y[j], acc[i][j]);
+    }
+    mfma_settle();
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s += acc[i][j][0];
+    if (sink != nullptr && __float_as_uint(s) == 0x7fc12345u) *sink = 1;      // a NaN payload the products never make
+}
+
 // Pure streaming read with the access pattern of the GeMV kernels (1 KiB tiles, 16 bytes per
 // lane, non-temporal, U loads in flight per wave): measures what the memory system delivers to
 // a kernel that does nothing else.  The xor of everything read is compared with a value the
@@ -265,6 +302,14 @@ int mlk_stream_read(const void *src, int64_t nbytes, int block_dim_x, int workgr
     MLK_REQUIRE(tiles % workgroups == 0, "stream_read: the workgroup count must divide the number of 1 KiB tiles");
     stream_read_kernel<4><<<workgroups, block_dim_x, 0, (hipStream_t)stream>>>((const u32x4 *)src, tiles / workgroups,
                                                                               (uint32_t *)sink);
+    MLK_LAUNCH_CHECK();
+    return MLK_OK;
+}
+
+int mlk_mfma_probe(const void *a, const void *b, int iters, int workgroups, void *sink, void *stream) {
+    MLK_REQUIRE(a && b, "mfma_probe: null pointer");
+    MLK_REQUIRE(iters >= 0 && workgroups >= 1, "mfma_probe: iterations >= 0, at least one workgroup");
+    mfma_probe_kernel<<<workgroups, 512, 0, (hipStream_t)stream>>>((const u32x4 *)a, (const u32x4 *)b, iters, (uint32_t *)sink);
     MLK_LAUNCH_CHECK();
     return MLK_OK;
 }
