@@ -428,6 +428,191 @@ __global__ void __launch_bounds__(512) gemm_panel8_kernel(PanelArgs p) {
     panel_finish<T, PR, TB, 8, 2>(p, acc, rg0, tok0 + wt * 128, SK, sk, rt, tt, wave, lane, reinterpret_cast<int *>(win));
 }
 
+// The same panel for soft-FP8 weights.  The fp8 tiles (512 bytes) land in a small ring of their own (three slabs of
+// 8 KiB behind the four bf16 slabs: 152 KiB in all); every wave widens the two tiles it fetched itself, two slabs ahead of
+// their use, lane by lane (8 bytes in, 16 bytes out at the same lane's place: the tile order does not change) into the
+// bf16 slab, so that each weight is widened once per workgroup and the multiplying loop is the 16-bit one.  Per slab and
+// wave: two token-chunk loads, one fp8 load (its two tiles, 32 lanes each), two 8-byte LDS reads, 32 conversion
+// instructions, two 16-byte LDS writes, sixteen products.
+constexpr int kP8RawSlab = 512;                                // granules of a slab of fp8 tiles
+constexpr size_t kP8Fp8LdsBytes = (size_t)(4 * kP8Slab + 3 * kP8RawSlab) * 16;
+
+__device__ __forceinline__ void p8_issue_fp8(const uint8_t *a_panel, const uint16_t *b, uint32_t a_voff, const uint32_t *b_voff,
+                                             int wave, int slab_b, int buf_b, int slab_a, int buf_a) {
+    extern __shared__ u32x4 win[];
+    __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc((void *)a_panel, 0, 0xffffffffu, 0x00020000);
+    __amdgpu_buffer_rsrc_t rs_b = __builtin_amdgcn_make_buffer_rsrc((void *)b, 0, 0xffffffffu, 0x00020000);
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_b, win + buf_b * kP8Slab + 1024 + (2 * wave + i) * 64, 16, b_voff[i], slab_b * 64, 0, 0);
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, win + 4 * kP8Slab + buf_a * kP8RawSlab + 2 * wave * 32, 16, a_voff, slab_a * 512, 0, 0);
+}
+
+template <class T>
+__global__ void __launch_bounds__(512) gemm_panel8_fp8_kernel(PanelArgs p) {
+    extern __shared__ u32x4 win[];
+    constexpr int PR = 2, TB = 4;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wr = wave & 3, wt = wave >> 2;
+    const int xcd = blockIdx.x & 7;
+    int u = blockIdx.x >> 3;
+    int SK, sk, tt, rt;
+    if (p.band > 0) {
+        const int TT = p.token_tiles, groups8 = (p.row_tiles + 7) >> 3, RB = p.band, TC = p.chunk;
+        const int band = u / (RB * TT);
+        const int nb = min(RB, groups8 - band * RB);
+        const int v = u - band * RB * TT;
+        const int c = v / (nb * TC);
+        const int tc = min(TC, TT - c * TC);
+        const int w = v - c * nb * TC;
+        SK = 1, sk = 0;
+        tt = c * TC + w % tc;
+        rt = (band * RB + w / tc) * 8 + xcd;
+    } else {
+        const int whole_wgs = p.whole_groups * p.token_tiles;
+        const bool sliced = u >= whole_wgs;
+        SK = sliced ? p.SK : 1;
+        if (sliced) u -= whole_wgs;
+        tt = u % p.token_tiles;
+        u /= p.token_tiles;
+        sk = u % SK;
+        rt = ((sliced ? p.whole_groups : 0) + u / SK) * 8 + xcd;
+    }
+    if (rt >= p.row_tiles) return;
+
+    const int groups = p.N >> 4;
+    const int rgp = rt * 16;
+    const int rg0 = rgp + wr * 4;
+    const int tok0 = tt * 256;
+    const int nwin_total = p.K / 64;
+    const int wbeg = (int)((long long)sk * nwin_total / SK);
+    const int slab0 = 2 * wbeg;
+    const int nslab = 2 * ((int)((long long)(sk + 1) * nwin_total / SK) - wbeg);
+    const int scale_cols = (p.K + 127) >> 7;
+
+    // this wave fetches and widens the tiles of row groups rgp + 2 wave, + 1 (rows past N: the last row group)
+    const uint8_t *a_panel = p.A + (size_t)rgp * p.K * 16;
+    const int rga = min(rgp + 2 * wave, groups - 1), rgb = min(rgp + 2 * wave + 1, groups - 1);
+    const uint32_t a_voff = (uint32_t)((lane >> 5 ? rgb : rga) - rgp) * (uint32_t)p.K * 16u + (lane & 31) * 16;
+    const ScaleRow srow = load_scale_row(p.scale ? p.scale + (size_t)(rga >> 3) * scale_cols : nullptr, scale_cols, lane);
+    uint32_t b_voff[2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+        const int t = lane >> 2, oct = (lane & 3) ^ ((t >> 2) & 3);
+        const int tok = min(tok0 + (2 * wave + i) * 16 + t, p.M - 1);
+        b_voff[i] = (uint32_t)tok * (uint32_t)p.K * 2u + oct * 16;
+    }
+    const int g = lane >> 5, i32 = lane & 31, t16 = i32 & 15, hi = i32 >> 4;
+    const int a_idx = (wr * 4 + hi) * 64 + g * 16 + t16;
+    const int b_idx = 1024 + (wt * 8 + hi) * 64 + 4 * t16 + (g ^ ((t16 >> 2) & 3));
+
+    f32x16 acc[PR][TB];
+#pragma unroll
+    for (int pr = 0; pr < PR; ++pr)
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+            for (int e = 0; e < 16; ++e) acc[pr][tb][e] = 0.f;
+
+    u32x4 a0[PR], a1[PR], b0[TB], b1[TB];
+    auto rd = [&](u32x4 (&a)[PR], u32x4 (&b)[TB], int buf, int hs) {
+        const u32x4 *src = win + buf * kP8Slab;
+#pragma unroll
+        for (int pr = 0; pr < PR; ++pr) a[pr] = src[a_idx + 128 * pr + hs * 32];
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb) b[tb] = src[(b_idx ^ (hs * 2)) + 128 * tb];
+    };
+    auto mm = [&](const u32x4 (&a)[PR], const u32x4 (&b)[TB]) {
+#pragma unroll
+        for (int tb = 0; tb < TB; ++tb)
+#pragma unroll
+            for (int pr = 0; pr < PR; ++pr) acc[pr][tb] = T::mfma32(a[pr], b[tb], acc[pr][tb]);
+    };
+    // widen this wave's two tiles of slab `slab` (counted from k = 0) from raw buffer rb into bf16 slab buffer `buf`
+    auto widen = [&](int slab, int rb, int buf) {
+        const float sc = scale_at(srow, slab >> 2);
+        const u32x2 *raw = reinterpret_cast<const u32x2 *>(win + 4 * kP8Slab + rb * kP8RawSlab + 2 * wave * 32);
+        u32x4 *dst = win + buf * kP8Slab + 2 * wave * 64;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const u32x2 f = raw[i * 64 + lane];
+            uint32_t x0, x1, x2, x3;
+            fp8x4_to_bf16x4(f[0], sc, x0, x1);
+            fp8x4_to_bf16x4(f[1], sc, x2, x3);
+            dst[i * 64 + lane] = u32x4{x0, x1, x2, x3};
+        }
+    };
+    // Order of this wave's loads: chunks(0) raw(0) chunks(1) raw(1) chunks(2) raw(2) | raw(3) | then per trip s: chunks(s + 3)
+    // raw(s + 4).  Slabs past the end of the slice are fetched (and widened) as copies of its last slab and never multiplied.
+    const int last = slab0 + nslab - 1;
+#pragma unroll
+    for (int i = 0; i < 3; ++i) p8_issue_fp8(a_panel, p.B, a_voff, b_voff, wave, min(slab0 + i, last), i, min(slab0 + i, last), i);
+    wait_vmcnt_le<3>();                                        // chunks and tiles of slabs 0 and 1 have landed
+    widen(min(slab0, last), 0, 0);
+    widen(min(slab0 + 1, last), 1, 1);
+    {   // raw(3) into the raw buffer that slab 0 has left
+        __amdgpu_buffer_rsrc_t rs_a = __builtin_amdgcn_make_buffer_rsrc((void *)a_panel, 0, 0xffffffffu, 0x00020000);
+        __builtin_amdgcn_raw_ptr_buffer_load_lds(rs_a, win + 4 * kP8Slab + 0 * kP8RawSlab + 2 * wave * 32, 16, a_voff,
+                                                 min(slab0 + 3, last) * 512, 0, 0);
+    }
+    __builtin_amdgcn_s_waitcnt(0xc07f);                        // lgkmcnt(0): the widened tiles are written
+    bare_barrier();
+    rd(a0, b0, 0, 0);
+    int cur = 0, rcur = 0;                                     // ring buffer of slab s, raw buffer of slab s
+    for (int s = 0; s < nslab; ++s) {
+        const int nxt = (cur + 1) & 3, nx2 = (cur + 2) & 3, prv = (cur + 3) & 3;
+        const int r1 = rcur == 2 ? 0 : rcur + 1, r2 = rcur == 0 ? 2 : rcur - 1;      // raw buffers of slabs s + 1 (= s + 4), s + 2
+        p8_issue_fp8(a_panel, p.B, a_voff, b_voff, wave, min(slab0 + s + 3, last), prv, min(slab0 + s + 4, last), r1);
+        // the tiles of slab s + 2: everything younger than them may still be in flight (four loads in the first trip,
+        // where raw(3) went out alone; six from then on)
+        if (s == 0) wait_vmcnt_le<4>();
+        else wait_vmcnt_le<6>();
+        // the fp8 tiles are read first, widened between the products of the first half step and written after them
+        const float sc = scale_at(srow, min(slab0 + s + 2, last) >> 2);
+        const u32x2 *raw = reinterpret_cast<const u32x2 *>(win + 4 * kP8Slab + r2 * kP8RawSlab + 2 * wave * 32);
+        const u32x2 f0 = raw[lane], f1 = raw[64 + lane];
+        rd(a1, b1, cur, 1);
+        u32x4 w0, w1;
+        {
+            uint32_t x0, x1, x2, x3;
+            fp8x4_to_bf16x4(f0[0], sc, x0, x1);
+            fp8x4_to_bf16x4(f0[1], sc, x2, x3);
+            w0 = u32x4{x0, x1, x2, x3};
+            fp8x4_to_bf16x4(f1[0], sc, x0, x1);
+            fp8x4_to_bf16x4(f1[1], sc, x2, x3);
+            w1 = u32x4{x0, x1, x2, x3};
+        }
+        mm(a0, b0);
+        {
+            u32x4 *dst = win + nx2 * kP8Slab + 2 * wave * 64;
+            dst[lane] = w0;
+            dst[64 + lane] = w1;
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, 8, 0);       // the LDS reads
+        __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+#pragma unroll
+        for (int m = 2; m < 8; ++m) {
+            __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);   // six conversion instructions
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x200, 2, 0);       // the two LDS writes
+        __builtin_amdgcn_sched_barrier(0);
+        rd(a0, b0, nxt, 0);
+        mm(a1, b1);
+        __builtin_amdgcn_sched_barrier(0);
+        wait_vmcnt_le<4>();                                    // this wave's chunks of slab s + 2 have landed
+        __builtin_amdgcn_s_waitcnt(0xc07f);                    // and its widened tiles are written
+        bare_barrier();
+        cur = nxt;
+        rcur = r1;
+    }
+    __builtin_amdgcn_s_waitcnt(0);
+    mfma_settle();
+    __syncthreads();
+    panel_finish<T, PR, TB, 8, 2>(p, acc, rg0, tok0 + wt * 128, SK, sk, rt, tt, wave, lane, reinterpret_cast<int *>(win));
+}
+
 // Tokens per panel when the caller leaves the choice open.  Workgroups run one per CU in rounds; a 256-token panel
 // takes 1.3 to 1.5 times as long as a 128-token one for 16-bit weights (eight-wave kernel) and 1.84 times for soft-FP8
 // ones (measured), so the width with the cheaper sum of rounds wins.
@@ -516,28 +701,27 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
         }                                                                                                          \
         gemm_panel_kernel<TT, F8, TBB, PRR><<<grid, 256, lds, s>>>(p);                                                  \
     } while (0)
-    if (width == 256 && a_kind != MLK_FP8_E4M3) {
+    if (width == 256) {
         // eight waves, operands through LDS
-#define MLK_PANEL8(TT)                                                                                                 \
+#define MLK_PANEL8(KERNEL, LDS)                                                                                        \
     do {                                                                                                           \
         static bool ready_on[64] = {};                                                                             \
         bool &ready = ready_on[dev & 63];                                                                          \
         if (!ready) {                                                                                              \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&gemm_panel8_kernel<TT>),            \
-                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)kP8LdsBytes);     \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(&KERNEL),                            \
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)(LDS));           \
             if (e != hipSuccess) return fail(MLK_ERR_LAUNCH, hipGetErrorString(e));                                \
             ready = true;                                                                                          \
         }                                                                                                          \
-        gemm_panel8_kernel<TT><<<grid, 512, kP8LdsBytes, s>>>(p);                                                  \
+        KERNEL<<<grid, 512, LDS, s>>>(p);                                                                          \
     } while (0)
         const bool whole = p.SK == 1 && p.whole_groups == 0;
         p.band = whole ? 8 : 0;
         p.chunk = 4;
-        if (a_kind == MLK_F16) MLK_PANEL8(F16);
-        else MLK_PANEL8(BF16);
+        if (a_kind == MLK_FP8_E4M3) MLK_PANEL8(gemm_panel8_fp8_kernel<BF16>, kP8Fp8LdsBytes);
+        else if (a_kind == MLK_F16) MLK_PANEL8(gemm_panel8_kernel<F16>, kP8LdsBytes);
+        else MLK_PANEL8(gemm_panel8_kernel<BF16>, kP8LdsBytes);
 #undef MLK_PANEL8
-    } else if (width == 256) {
-        MLK_PANEL(BF16, true, 8, 2);
     } else if (rows == 256 && a_kind == MLK_FP8_E4M3 && (p.SK == 1 || p.whole_groups > 0)) {
         // soft-FP8, panels computed whole (or only the last round's sliced): the loop that prefetches through LDS, two
         // workgroups per CU (28672 x 8192 at 1024 tokens: 616 -> 474 us); fully sliced grids and 16-bit weights stay on

@@ -97,3 +97,17 @@ def test_stream_read_probe(mlk):
     torch.cuda.synchronize()
     assert torch.equal(buf, keep)
     assert lib.mlk_stream_read(buf.data_ptr(), buf.numel(), 256, 1000, None, st) == -1   # 8192 tiles % 1000 != 0
+
+
+def test_mfma_probe(mlk):
+    """The matrix-core yardstick runs, writes nothing, and refuses null operands."""
+    from muxi_native_layout_kernels_amd import _lib
+    lib = _lib.load()
+    a = torch.randn((64 * 1024,), device="cuda").to(torch.bfloat16)
+    b = torch.randn((64 * 1024,), device="cuda").to(torch.bfloat16)
+    keep = (a.clone(), b.clone())
+    st = torch.cuda.current_stream().cuda_stream
+    assert lib.mlk_mfma_probe(a.data_ptr(), b.data_ptr(), 10, 8, None, st) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(a, keep[0]) and torch.equal(b, keep[1])
+    assert lib.mlk_mfma_probe(None, b.data_ptr(), 10, 8, None, st) == -1
