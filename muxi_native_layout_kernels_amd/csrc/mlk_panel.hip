@@ -262,6 +262,47 @@ __global__ void __launch_bounds__(256, 2) gemm_panel_lds_kernel(PanelArgs p) {
     panel_finish<T, PR, TB, kTileWaves, 2>(p, acc, rg0, tok0, SK, sk, rt, tt, wave, lane, reinterpret_cast<int *>(win));
 }
 
+// Output of an eight-wave panel that is computed whole: every wave turns its 64 rows x 128 tokens around in LDS (the ring
+// is free by then; 144 bytes per token, so that the 8-byte pieces of 32 tokens meet each bank at most twice) and stores
+// whole 128-byte lines, eight tokens per instruction.  Stored straight from the accumulators, a lane's four rows of one
+// token are 8 bytes in a line that fifteen other instructions complete: 67 MB of output took 23 us that way.
+constexpr int kP8OutPitch = 144;                               // bytes per token in the turn-around buffer
+constexpr size_t kP8OutBytes = (size_t)8 * 128 * kP8OutPitch;
+template <class T>
+__device__ __forceinline__ void p8_store_panel(const PanelArgs &p, f32x16 (&acc)[2][4], int rg0, int tok0, int wave, int lane,
+                                               u32x4 *win) {
+    uint8_t *buf = reinterpret_cast<uint8_t *>(win) + (size_t)wave * 128 * kP8OutPitch;
+    const int half = lane >> 5, c32 = lane & 31;
+    const int n0 = rg0 * 16;                                   // first of the wave's 64 rows
+#pragma unroll
+    for (int pr = 0; pr < 2; ++pr)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const int row = pr * 32 + 8 * g + 4 * half;        // of the wave's 64
+            float bias[4] = {0.f, 0.f, 0.f, 0.f};
+            if (p.bias && n0 + row < p.N) {
+#pragma unroll
+                for (int i = 0; i < 4; ++i) bias[i] = T::to_f32(p.bias[n0 + row + i]);
+            }
+#pragma unroll
+            for (int tb = 0; tb < 4; ++tb) {
+                u32x2 o;
+                o[0] = T::from_f32(p.alpha * acc[pr][tb][4 * g] + bias[0]) | (T::from_f32(p.alpha * acc[pr][tb][4 * g + 1] + bias[1]) << 16);
+                o[1] = T::from_f32(p.alpha * acc[pr][tb][4 * g + 2] + bias[2]) | (T::from_f32(p.alpha * acc[pr][tb][4 * g + 3] + bias[3]) << 16);
+                *reinterpret_cast<u32x2 *>(buf + (tb * 32 + c32) * kP8OutPitch + row * 2) = o;
+            }
+        }
+    // lane 8 t + q: 16 bytes (8 rows) q of token t of each group of eight tokens
+    const int t8 = lane >> 3, q = lane & 7;
+    const bool rows_ok = n0 + q * 8 < p.N;
+#pragma unroll
+    for (int it = 0; it < 16; ++it) {
+        const int token = it * 8 + t8;
+        const u32x4 v = *reinterpret_cast<const u32x4 *>(buf + token * kP8OutPitch + q * 16);
+        if (rows_ok && tok0 + token < p.M) *reinterpret_cast<u32x4 *>(p.C + (size_t)(tok0 + token) * p.N + n0 + q * 8) = v;
+    }
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // 256 x 256 panels of 16-bit weights: eight waves, both operands through LDS, fetched with loads that write LDS directly.
 //
@@ -283,7 +324,7 @@ __global__ void __launch_bounds__(256, 2) gemm_panel_lds_kernel(PanelArgs p) {
 // are read before that barrier, so no wave stands idle behind it.  The barrier is the bare instruction: the fence that
 // comes with __syncthreads() would wait for every load in flight.
 constexpr int kP8Slab = 2048;                                  // 16-byte granules of a slab: 1024 of weights, 1024 of tokens
-constexpr size_t kP8LdsBytes = (size_t)4 * kP8Slab * 16;
+constexpr size_t kP8RingBytes = (size_t)4 * kP8Slab * 16;
 
 // the four loads of one wave for slab `slab` (counted from k = 0) into ring buffer `buf`
 __device__ __forceinline__ void p8_issue(const uint8_t *a_panel, const uint16_t *b, const uint32_t (&a_soff)[2],
@@ -425,7 +466,8 @@ __global__ void __launch_bounds__(512) gemm_panel8_kernel(PanelArgs p) {
     __builtin_amdgcn_s_waitcnt(0);                             // nothing may still be writing LDS when the ring is given up
     mfma_settle();
     __syncthreads();
-    panel_finish<T, PR, TB, 8, 2>(p, acc, rg0, tok0 + wt * 128, SK, sk, rt, tt, wave, lane, reinterpret_cast<int *>(win));
+    if (SK == 1) p8_store_panel<T>(p, acc, rg0, tok0 + wt * 128, wave, lane, win);
+    else panel_finish<T, PR, TB, 8, 2>(p, acc, rg0, tok0 + wt * 128, SK, sk, rt, tt, wave, lane, reinterpret_cast<int *>(win));
 }
 
 // The same panel for soft-FP8 weights.  The fp8 tiles (512 bytes) land in a small ring of their own (three slabs of
@@ -610,7 +652,8 @@ __global__ void __launch_bounds__(512) gemm_panel8_fp8_kernel(PanelArgs p) {
     __builtin_amdgcn_s_waitcnt(0);
     mfma_settle();
     __syncthreads();
-    panel_finish<T, PR, TB, 8, 2>(p, acc, rg0, tok0 + wt * 128, SK, sk, rt, tt, wave, lane, reinterpret_cast<int *>(win));
+    if (SK == 1) p8_store_panel<T>(p, acc, rg0, tok0 + wt * 128, wave, lane, win);
+    else panel_finish<T, PR, TB, 8, 2>(p, acc, rg0, tok0 + wt * 128, SK, sk, rt, tt, wave, lane, reinterpret_cast<int *>(win));
 }
 
 // Tokens per panel when the caller leaves the choice open.  Workgroups run one per CU in rounds; a 256-token panel
@@ -718,9 +761,12 @@ int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int
         const bool whole = p.SK == 1 && p.whole_groups == 0;
         p.band = whole ? 8 : 0;
         p.chunk = 4;
-        if (a_kind == MLK_FP8_E4M3) MLK_PANEL8(gemm_panel8_fp8_kernel<BF16>, kP8Fp8LdsBytes);
-        else if (a_kind == MLK_F16) MLK_PANEL8(gemm_panel8_kernel<F16>, kP8LdsBytes);
-        else MLK_PANEL8(gemm_panel8_kernel<BF16>, kP8LdsBytes);
+        // LDS: the ring, or the turn-around buffer of the output if that is larger
+        constexpr size_t lds16 = kP8RingBytes > kP8OutBytes ? kP8RingBytes : kP8OutBytes;
+        constexpr size_t lds8 = kP8Fp8LdsBytes > kP8OutBytes ? kP8Fp8LdsBytes : kP8OutBytes;
+        if (a_kind == MLK_FP8_E4M3) MLK_PANEL8(gemm_panel8_fp8_kernel<BF16>, lds8);
+        else if (a_kind == MLK_F16) MLK_PANEL8(gemm_panel8_kernel<F16>, lds16);
+        else MLK_PANEL8(gemm_panel8_kernel<BF16>, lds16);
 #undef MLK_PANEL8
     } else if (rows == 256 && a_kind == MLK_FP8_E4M3 && (p.SK == 1 || p.whole_groups > 0)) {
         // soft-FP8, panels computed whole (or only the last round's sliced): the loop that prefetches through LDS, two
