@@ -40,6 +40,9 @@ where the weights are small, HBM traffic from hardware counters where a
 profile under profiles/ holds it, and the CPU baseline of that configuration:
 the reference's CPU-runnable torch path (a library linear on the un-packed
 weights, or its dense MoE loop) timed on the host cores on a bounded sample.
+The prefill lines ("next: prefill ...") report TFLOP/s and the fraction of the 2.5 PFLOP/s MFMA peak, the vendor BLAS
+on un-packed weights of the same shape (`blas_us`) and `mfma_only_tflops`: what a loop of nothing but the MFMA instruction
+sustains in the same run on operand values drawn like the benchmark's (the power limit, not the issue rate, sets it).
 
 `eager_calls` holds the public Python API timed the way the reference's own
 scripts time it: the wall clock around 1000 eager calls (300 for the fused MoE),
