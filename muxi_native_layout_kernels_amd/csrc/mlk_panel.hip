@@ -680,7 +680,7 @@ size_t panel_partial_bytes(int m, int n, int sk) {
 int launch_panel(const void *a, const void *b, void *c, int m, int n, int k, int a_kind, float alpha, const void *bias,
                  const float *scale, int width, int rows, int sk, bool last_round_only, void *counters,
                  size_t counter_bytes, void *partial, size_t partial_bytes, hipStream_t s) {
-    PanelArgs p;
+    PanelArgs p = {};
     p.A = (const uint8_t *)a;
     p.B = (const uint16_t *)b;
     p.C = (uint16_t *)c;

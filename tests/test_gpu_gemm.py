@@ -220,6 +220,30 @@ def test_gemm_panel_kernel_last_round_slices_soft_fp8(mlk):
     assert_close(c, ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), b), RTOL, ATOL, "panel fp8, last round sliced")
 
 
+@pytest.mark.parametrize("fp8", [False, True])
+def test_gemm_panel_kernel_band_and_chunk_mapping(mlk, fp8):
+    """256 x 256 panels computed whole: the workgroup ids walk bands of eight groups of row tiles in chunks of four token
+    tiles.  73 row tiles = ten groups (a band of eight and one of two, the last group with one row tile) and six token
+    tiles (a chunk of four and one of two, the last tile ragged): every output element is checked."""
+    n, k, m = 18560, 256, 1300
+    b = randn((m, k), torch.bfloat16, 1.0, 292)
+    if fp8:
+        codes = fp8_codes((n, k), 293)
+        g = torch.Generator().manual_seed(294)
+        scale = (torch.rand((n // 128, k // 128), generator=g) * 0.02 + 0.001).float()
+        c = mlk.gemm_layoutA_soft_fp8_wapper(pack_a(codes).cuda(), scale.cuda(), b.cuda(), n, m, k, kernelParam1=4,
+                                             kernelParam2=2, kernelParam3=1, kernelId=3)
+        want = ogemm.softfp8_linear_expected(codes.numpy(), scale.numpy(), b)
+    else:
+        w = randn((n, k), torch.bfloat16, 0.05, 291)
+        bias = randn((1, n), torch.bfloat16, 1.0, 295)
+        c = mlk.gemm_layoutA_wapper(pack_a(w).cuda(), b.cuda(), n, m, k, alpha=0.5, kernelParam1=4, kernelParam2=2,
+                                    kernelParam3=1, kernelId=3, bias=bias.cuda())
+        want = ogemm.linear_expected(w, b, 0.5, bias)
+    assert c.shape == (m, n)
+    assert_close(c, want, RTOL, ATOL, "band / chunk mapping fp8=%s" % fp8)
+
+
 def test_gemm_panel_kernel_is_the_wide_default(mlk):
     """Above 64 tokens the heuristic for unscanned shapes picks the panel kernel; a K that is no
     multiple of 128 keeps the row-shared kernel, and the panel kernel refuses it when asked for by id."""
