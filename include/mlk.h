@@ -67,6 +67,8 @@ const char *mlk_last_error(void);
  *         expert's weights, 1..8 (default 0 = sized from the expected load of an expert)
  *   id 9  fused MoE, soft-FP8 weights, more than 64 tokens per pass over an expert: 1 keeps the row-shared
  *         kernels instead of the panel kernels (default 0)
+ *   10    fused MoE, panel kernels: shape of the down projection, K slices (1..8) + 16 x (two workgroups per
+ *         CU on the short LDS ring); 0 (default) = chosen from the sizes and the device's CU count
  * The MoE scan script (kernel_args_scan/moe_scan.py) sweeps ids 2..5, 7 and 8.
  * No counterpart in the reference. */
 void mlk_set_tunable(int id, int value);
@@ -291,8 +293,9 @@ int mlk_fused_moe(const void *w1, const void *w2, const void *x, const void *log
  * kernels after the alignment kernel, 3 row-shared kernels, 4 panel kernels: soft-FP8 weights with more than 64
  * tokens per pass over an expert), out[1] = token blocks per task, out[2] = upper bound of the task list,
  * out[3] = row groups per wave and out[4] = K slices of the down projection, out[5] = waves and out[6] = dynamic
- * LDS bytes of the decode down kernel (families 1, 2), out[7] = its static LDS bytes.  Everything follows from
- * the sizes alone except out[4] of family 4, which also depends on the number of compute units of the current
+ * LDS bytes of the decode down kernel (families 1, 2; for family 4 out[5] = workgroups per CU the down kernel is
+ * built for, 1 or 2), out[7] = its static LDS bytes.  Everything follows from
+ * the sizes alone except out[4] and out[5] of family 4, which also depend on the number of compute units of the current
  * device: for that family the call asks the HIP runtime for it (which initialises the runtime) and assumes 256
  * where there is no GPU, so a plan made on a host without a GPU can name another slice count than a launch on a
  * device with a different CU count uses.  For tests and the tuning scripts; no counterpart in the reference. */

@@ -1315,15 +1315,36 @@ static int launch_moe_cb(const MoeArgs &a, int cb, int max_tasks, bool inline_al
     }
 }
 
-extern template int launch_moe_panel<BF16, true>(const MoeArgs &, int, int, float *, int, hipStream_t);
+extern template int launch_moe_panel<BF16, true>(const MoeArgs &, int, int, float *, int, bool, hipStream_t);
 
-// K slices of the panel down projection: its grid is (H / 256 row tiles, tasks, slices); slice K while the grid
-// holds fewer than one and a half workgroups per CU and a slice keeps at least four 128-wide k windows.
-static int moe_panel_down_slices(int hidden, int inter, int max_tasks) {
+// Shape of the panel down projection: its grid is (H / 256 row tiles, tasks, K slices), and its kernel comes with a
+// short LDS ring (two workgroups per CU, two waves per SIMD) and a long one (one per CU).  Two per CU pay when the
+// grid fills them: `pairs` when K slices of at least four 128-wide k windows bring the expected grid (one task per
+// active expert; the task list's upper bound counts the tasks a skewed routing adds) to two workgroups per CU
+// (Mixtral shape, 256 tokens: 16 x 8 x 4 workgroups, 118 us against 140 us with one per CU and two slices, and 177 us
+// with two per CU and two slices, which leaves half the CUs idle).  Otherwise one per CU: slice K while the grid's
+// upper bound holds fewer than one and a half workgroups per CU.
+// Experiment switch 10: slices + 16 x pairs, in place of this choice.
+static void moe_panel_down_shape(int hidden, int inter, int active, int max_tasks, int *slices, bool *pairs) {
     const int row_tiles = hidden / 256, windows = inter / 128, cus = device_cus();
+    if (g_tunable[10] > 0) {
+        *slices = g_tunable[10] & 15;
+        if (*slices < 1) *slices = 1;
+        if (*slices > kMoeMaxKSlices) *slices = kMoeMaxKSlices;
+        if (*slices > windows) *slices = windows;
+        *pairs = (g_tunable[10] >> 4) != 0;
+        return;
+    }
     int skd = 1;
+    while (skd < kMoeMaxKSlices && row_tiles * active * skd < 2 * cus && windows / (skd * 2) >= 4) skd *= 2;
+    *pairs = row_tiles * active * skd >= 2 * cus;
+    if (*pairs) {
+        *slices = skd;
+        return;
+    }
+    skd = 1;
     while (skd < kMoeMaxKSlices && row_tiles * max_tasks * skd * 2 < cus * 3 && windows / (skd * 2) >= 4) skd *= 2;
-    return skd;
+    *slices = skd;
 }
 // blocks of 32 tokens in a panel for tasks of up to cb blocks of 16
 static int moe_panel_tb32(int cb) { return (cb + 1) / 2 > 4 ? 4 : (cb + 1) / 2; }
@@ -1340,7 +1361,8 @@ struct MoePlan {
     int max_tasks;    // upper bound of the task list (grid dimension)
     int down_r;       // down projection: row groups per wave
     int down_slices;  // down projection: K slices across workgroups
-    int down_wk;      // decode down kernel: waves per workgroup
+    bool down_pairs;  // panel down projection: two workgroups per CU (shorter LDS ring)
+    int down_wk;      // decode down kernel: waves per workgroup; panel down kernel: workgroups per CU
     size_t down_lds;  // decode down kernel: dynamic LDS bytes
 };
 static MoePlan moe_plan(int tc, int n_experts, int topk, int hidden, int inter, bool fp8) {
@@ -1360,7 +1382,8 @@ static MoePlan moe_plan(int tc, int n_experts, int topk, int hidden, int inter, 
     if (!inline_align && moe_tile_path() && moe_panel_path(pl.cb, hidden, fp8)) {
         pl.path = kMoePathPanel;
         pl.down_r = 4;
-        pl.down_slices = moe_panel_down_slices(hidden, inter, pl.max_tasks);
+        moe_panel_down_shape(hidden, inter, active, pl.max_tasks, &pl.down_slices, &pl.down_pairs);
+        pl.down_wk = pl.down_pairs ? 2 : 1;
         return pl;
     }
     if (!inline_align && pl.cb >= 2 && (moe_tile_path() || pl.cb > 4)) {
@@ -1602,7 +1625,7 @@ static int experts_compute_impl(const void *w1, const void *w2, const void *x, i
         if (pl.path == kMoePathPanel) {
             const int tb32 = moe_panel_tb32(cb), skd = pl.down_slices;
             const dim3 cgrid(tc, (hidden + 1023) / 1024);
-            rc = launch_moe_panel<BF16, true>(a, tb32, max_tasks, ws.obuf, skd, s);
+            rc = launch_moe_panel<BF16, true>(a, tb32, max_tasks, ws.obuf, skd, pl.down_pairs, s);
             if (rc != MLK_OK) return rc;
             moe_combine_kernel<BF16><<<cgrid, 256, 0, s>>>(ws.obuf, a.Y, a.topk_ids, a.experts_map, topk, hidden, n_experts, skd);
             MLK_LAUNCH_CHECK();

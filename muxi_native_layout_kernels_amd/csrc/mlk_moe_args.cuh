@@ -36,6 +36,6 @@ struct MoeArgs {
 // is kept row-major [slot][I] (slot = position in the alignment), the weighted products go to obuf
 // [routed pair][K slice][H] for moe_combine_kernel.  Needs H % 256 == 0.
 template <class T, bool FP8>
-int launch_moe_panel(const MoeArgs &a, int tb32, int max_tasks, float *obuf, int skd, hipStream_t s);
+int launch_moe_panel(const MoeArgs &a, int tb32, int max_tasks, float *obuf, int skd, bool down_pairs, hipStream_t s);
 
 }  // namespace mlk

@@ -1,5 +1,6 @@
-// Fused MoE above 16 tokens per expert on the panel main loop (mlk_panel_loop.cuh): v_mfma_f32_32x32x16, weights
-// straight from the per-expert layout-A slabs, the task's token rows shared through LDS.
+// Fused MoE above 16 tokens per expert on the LDS-fed panel main loop (PanelLoopLds, mlk_panel_lds.cuh):
+// v_mfma_f32_32x32x16, weights from the per-expert layout-A slabs straight into an LDS ring, the task's token rows
+// shared through the same ring.
 //
 //   gate/up   grid (I / 128, tasks).  A wave owns 32 columns of the intermediate: one pair of row groups from the
 //             gate half of W1[expert] and the pair with the same index from the up half, so that gate and up of an
@@ -16,10 +17,9 @@
 // Where it is used: soft-FP8 weights with more than 64 tokens per pass over an expert.  There the weight stream is
 // half as long as with 16-bit weights and the matrix cores set the pace; the row-shared kernels (16x16x32
 // products, one wave per SIMD) reach about a fifth of their peak, this loop about two fifths (measured on the
-// Mixtral shape at 256 tokens: 549 us -> 424 us).  With 16-bit weights, and with fewer tokens per expert, the layer
-// is bound by the weight stream and the row-shared kernels are as fast or faster (they fit two or three workgroups
-// on a CU; this loop takes a whole register file), so only the soft-FP8 form is instantiated
-// (mlk_moe_panel_fp8.hip).
+// Mixtral shape at 256 tokens: 549 us -> 385 us).  With 16-bit weights, and with fewer tokens per expert, the layer
+// is bound by the weight stream and the row-shared kernels are as fast or faster (measured with this loop on bf16
+// weights: gate/up 362 against 325 us), so only the soft-FP8 form is instantiated (mlk_moe_panel_fp8.hip).
 #pragma once
 
 #include "mlk_moe_args.cuh"
@@ -30,16 +30,10 @@ namespace mlk {
 // Slabs of LDS per workgroup.  Gate/up: four (56 or 64 KiB), two workgroups per CU.  Down: six (84 or 96 KiB), one
 // workgroup per CU: its grid is about one workgroup per CU, and two of them on one CU while another CU idles cost
 // more than the second wave per SIMD brings (Mixtral shape, 256 tokens: 179 against 137 us).
-#ifndef MLK_GU_RING
-#define MLK_GU_RING 4
-#endif
-#ifndef MLK_GU_OCC
-#define MLK_GU_OCC 2
-#endif
-constexpr int kMoeGateUpRing = MLK_GU_RING, kMoeDownRing = 6;
+constexpr int kMoeGateUpRing = 4, kMoeDownRing = 6, kMoeDownPairRing = 4;
 
 template <class T, bool FP8, int TB>
-__global__ void __launch_bounds__(256, MLK_GU_OCC) moe_gate_up_panel_kernel(MoeArgs p) {
+__global__ void __launch_bounds__(256, 2) moe_gate_up_panel_kernel(MoeArgs p) {
     extern __shared__ u32x4 win[];
     const int task = blockIdx.y;
     if (task >= p.n_tasks[0]) return;
@@ -102,13 +96,13 @@ __global__ void __launch_bounds__(256, MLK_GU_OCC) moe_gate_up_panel_kernel(MoeA
     }
 }
 
-template <class T, bool FP8, int TB>
+template <class T, bool FP8, int TB, int RING>
 __global__ void __launch_bounds__(256, 2) moe_down_panel_kernel(MoeArgs p, float *__restrict__ O) {
     extern __shared__ u32x4 win[];
     const int task = blockIdx.y;
     if (task >= p.n_tasks[0]) return;
     const MoeTask tk = p.tasks[task];
-    using Loop = PanelLoopLds<T, FP8, TB, kMoeDownRing>;
+    using Loop = PanelLoopLds<T, FP8, TB, RING>;
     constexpr int WB = FP8 ? 1 : 2;
     const int tid = threadIdx.x, lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -176,26 +170,32 @@ static int panel_lds_attribute(K kernel, size_t lds, bool (&ready_on)[64]) {
 }
 
 template <class T, bool FP8, int TB>
-static int launch_moe_panel_tb(const MoeArgs &a, int max_tasks, float *obuf, int skd, hipStream_t s) {
+static int launch_moe_panel_tb(const MoeArgs &a, int max_tasks, float *obuf, int skd, bool down_pairs, hipStream_t s) {
     const size_t lds = PanelLdsShape<FP8, TB, kMoeGateUpRing>::lds_bytes;
     const size_t lds_down = PanelLdsShape<FP8, TB, kMoeDownRing>::lds_bytes;
-    static bool ready_gate[64] = {}, ready_down[64] = {};
+    const size_t lds_down2 = PanelLdsShape<FP8, TB, kMoeDownPairRing>::lds_bytes;
+    static bool ready_gate[64] = {}, ready_down[64] = {}, ready_down2[64] = {};
     int rc = panel_lds_attribute(&moe_gate_up_panel_kernel<T, FP8, TB>, lds, ready_gate);
     if (rc != MLK_OK) return rc;
-    rc = panel_lds_attribute(&moe_down_panel_kernel<T, FP8, TB>, lds_down, ready_down);
+    rc = panel_lds_attribute(&moe_down_panel_kernel<T, FP8, TB, kMoeDownRing>, lds_down, ready_down);
+    if (rc != MLK_OK) return rc;
+    rc = panel_lds_attribute(&moe_down_panel_kernel<T, FP8, TB, kMoeDownPairRing>, lds_down2, ready_down2);
     if (rc != MLK_OK) return rc;
     moe_gate_up_panel_kernel<T, FP8, TB><<<dim3(a.I / 128, max_tasks), 256, lds, s>>>(a);
     MLK_LAUNCH_CHECK();
-    moe_down_panel_kernel<T, FP8, TB><<<dim3(a.H / 256, max_tasks, skd), 256, lds_down, s>>>(a, obuf);
+    if (down_pairs)
+        moe_down_panel_kernel<T, FP8, TB, kMoeDownPairRing><<<dim3(a.H / 256, max_tasks, skd), 256, lds_down2, s>>>(a, obuf);
+    else
+        moe_down_panel_kernel<T, FP8, TB, kMoeDownRing><<<dim3(a.H / 256, max_tasks, skd), 256, lds_down, s>>>(a, obuf);
     MLK_LAUNCH_CHECK();
     return MLK_OK;
 }
 
 template <class T, bool FP8>
-int launch_moe_panel(const MoeArgs &a, int tb32, int max_tasks, float *obuf, int skd, hipStream_t s) {
+int launch_moe_panel(const MoeArgs &a, int tb32, int max_tasks, float *obuf, int skd, bool down_pairs, hipStream_t s) {
     switch (tb32) {
-        case 3: return launch_moe_panel_tb<T, FP8, 3>(a, max_tasks, obuf, skd, s);
-        case 4: return launch_moe_panel_tb<T, FP8, 4>(a, max_tasks, obuf, skd, s);
+        case 3: return launch_moe_panel_tb<T, FP8, 3>(a, max_tasks, obuf, skd, down_pairs, s);
+        case 4: return launch_moe_panel_tb<T, FP8, 4>(a, max_tasks, obuf, skd, down_pairs, s);
         default: return fail(MLK_ERR_INVALID, "moe: a panel holds 3 or 4 blocks of 32 tokens");
     }
 }

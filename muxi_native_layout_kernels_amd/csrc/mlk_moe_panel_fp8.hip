@@ -2,5 +2,5 @@
 #include "mlk_moe_panel.cuh"
 
 namespace mlk {
-template int launch_moe_panel<BF16, true>(const MoeArgs &, int, int, float *, int, hipStream_t);
+template int launch_moe_panel<BF16, true>(const MoeArgs &, int, int, float *, int, bool, hipStream_t);
 }

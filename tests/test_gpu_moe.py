@@ -225,6 +225,37 @@ def test_fused_moe_soft_fp8_panel_kernels(mlk, T, E, K, H, I):
     assert_close(y1, y2.double().cpu().numpy(), RTOL, ATOL, "panel kernels vs row-shared kernels")
 
 
+@pytest.mark.parametrize("switch", [1, 3, 17, 18, 20, 24])
+def test_fused_moe_soft_fp8_panel_down_shapes(mlk, switch):
+    """The panel down projection on the long LDS ring (one workgroup per CU) and on the short one (two per CU), in
+    1 to 8 K slices, each asked for through experiment switch 10 (slices + 16 x short ring) and checked against
+    the float64 statement."""
+    from muxi_native_layout_kernels_amd import _lib
+    import ctypes
+    lib = _lib.load()
+    T, E, K, H, I = 256, 8, 2, 256, 1024
+    plan = (ctypes.c_int32 * 8)()
+    lib.mlk_set_tunable(10, switch)
+    try:
+        assert lib.mlk_moe_plan(T, E, K, H, I, 2, ctypes.addressof(plan)) == 0 and plan[0] == 4
+        assert (plan[4], plan[5]) == (switch & 15, 2 if switch >> 4 else 1)
+        _moe_case(mlk, T, E, K, H, I, torch.bfloat16, 2300 + switch, fp8=True)
+    finally:
+        lib.mlk_set_tunable(10, 0)
+
+
+def test_fused_moe_soft_fp8_panel_down_two_per_cu(mlk):
+    """A shape whose down projection fills two workgroups per CU by itself (8 row tiles x 8 experts x 8 K slices):
+    the plan picks the short-ring kernel, and the result is checked against the float64 statement."""
+    from muxi_native_layout_kernels_amd import _lib
+    import ctypes
+    T, E, K, H, I = 256, 8, 2, 2048, 4096
+    plan = (ctypes.c_int32 * 8)()
+    assert _lib.load().mlk_moe_plan(T, E, K, H, I, 2, ctypes.addressof(plan)) == 0
+    assert plan[0] == 4 and (plan[4], plan[5]) == (8, 2), list(plan)
+    _moe_case(mlk, T, E, K, H, I, torch.bfloat16, 2400, fp8=True)
+
+
 def test_fused_moe_grouped_sigmoid_bias(mlk):
     E = 64
     bias = randn((E,), torch.bfloat16, 0.05, 9).abs()

@@ -194,6 +194,9 @@ def test_moe_plan_fits_the_workgroup_lds_for_every_token_count(E, K, H, I, kind)
         if p["path"] == 4:          # panel kernels: output rows in tiles of 256, at least four k windows per slice
             assert kind == 2 and p["cb"] >= 5 and H % 256 == 0 and 1 <= p["down_slices"] <= 8
             assert p["down_slices"] == 1 or (I // 128) // p["down_slices"] >= 4
+            assert p["down_wk"] in (1, 2)       # workgroups per CU the down kernel is built for
+            if p["down_wk"] == 2:               # two per CU only where the expected grid fills them (256 CUs assumed)
+                assert (H // 256) * min(E, T * K) * p["down_slices"] >= 512, (T, p)
         assert p["path"] != 0 or T == 1
 
 
@@ -213,6 +216,12 @@ def test_moe_plan_known_cases():
     # soft-FP8 with more than 64 tokens per pass over an expert: panel kernels, if the output rows tile in 256
     assert _plan(64, 8, 2, 4096, 14336, 2)["path"] == 3
     assert _plan(256, 8, 2, 4096, 14336, 2)["path"] == 4
+    # its down projection: 16 row tiles x 8 experts x 4 K slices = two workgroups on each of 256 CUs
+    mixtral = _plan(256, 8, 2, 4096, 14336, 2)
+    assert (mixtral["down_slices"], mixtral["down_wk"]) == (4, 2)
+    # a grid that cannot reach two per CU keeps one per CU: 4 row tiles x 8 experts x 8 slices = 256
+    small = _plan(256, 8, 2, 1024, 14336, 2)
+    assert small["path"] == 4 and small["down_wk"] == 1
     assert _plan(256, 8, 2, 4096 + 128, 14336, 2)["path"] == 3
     # 500 tokens run as 256 + 244: the plan of the first pass is what the query reports
     assert _plan(500, 256, 8, 7168, 256, 2) == _plan(256, 256, 8, 7168, 256, 2)
