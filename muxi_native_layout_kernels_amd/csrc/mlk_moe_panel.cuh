@@ -27,9 +27,11 @@
 
 namespace mlk {
 
-// Slabs of LDS per workgroup.  Gate/up: four (56 or 64 KiB), two workgroups per CU.  Down: six (84 or 96 KiB), one
-// workgroup per CU: its grid is about one workgroup per CU, and two of them on one CU while another CU idles cost
-// more than the second wave per SIMD brings (Mixtral shape, 256 tokens: 179 against 137 us).
+// Slabs of LDS per workgroup.  Gate/up: four (56 or 64 KiB), two workgroups per CU.  Down: the same where the host
+// found a K split that fills two workgroups per CU (moe_panel_down_shape in mlk_moe.hip), else six (84 or 96 KiB),
+// which keeps it to one workgroup per CU: on a grid of about one workgroup per CU, two of them on one CU while
+// another CU idles cost more than the second wave per SIMD brings (Mixtral shape, 256 tokens, 2 K slices: 177
+// against 137 us; 4 K slices on the short ring: 117 us).
 constexpr int kMoeGateUpRing = 4, kMoeDownRing = 6, kMoeDownPairRing = 4;
 
 template <class T, bool FP8, int TB>
