@@ -248,11 +248,12 @@ def test_gemm_panel_kernel_is_the_wide_default(mlk):
     """Above 64 tokens the heuristic for unscanned shapes picks the panel kernel; a K that is no
     multiple of 128 keeps the row-shared kernel, and the panel kernel refuses it when asked for by id."""
     from muxi_native_layout_kernels_amd import arg_selector
-    assert arg_selector.selector("layoutA_gemm").get_args((4096, 300, 1024))[0] == 3
-    assert arg_selector.selector("layoutA_soft_fp8_gemm").get_args((4096, 300, 1024))[0] == 3
-    assert arg_selector.selector("layoutA_gemm").get_args((4096, 300, 1088))[0] == 2
-    assert arg_selector.selector("layout_gemm").get_args((4096, 304, 1024))[0] == 2       # native operands
-    n, k, m = 4096, 1024, 300
+    # 4224 rows: a weight shape that no packaged table holds
+    assert arg_selector.selector("layoutA_gemm").get_args((4224, 300, 1024))[0] == 3
+    assert arg_selector.selector("layoutA_soft_fp8_gemm").get_args((4224, 300, 1024))[0] == 3
+    assert arg_selector.selector("layoutA_gemm").get_args((4224, 300, 1088))[0] == 2
+    assert arg_selector.selector("layout_gemm").get_args((4224, 304, 1024))[0] == 2       # native operands
+    n, k, m = 4224, 1024, 300
     w = randn((n, k), torch.bfloat16, 0.02, 98)
     b = randn((m, k), torch.bfloat16, 1.0, 99)
     c = mlk.gemm_layoutA_linear(pack_a(w).cuda(), b.cuda())
