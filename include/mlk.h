@@ -69,7 +69,7 @@ const char *mlk_last_error(void);
  *         kernels instead of the panel kernels (default 0)
  *   10    fused MoE, panel kernels: shape of the down projection, K slices (1..8) + 16 x (two workgroups per
  *         CU on the short LDS ring); 0 (default) = chosen from the sizes and the device's CU count
- * The MoE scan script (kernel_args_scan/moe_scan.py) sweeps ids 2..5, 7 and 8.
+ * The MoE scan script (kernel_args_scan/moe_scan.py) sweeps ids 2..5, 7, 8 and 10.
  * No counterpart in the reference. */
 void mlk_set_tunable(int id, int value);
 /* Experiment switches of the fused MoE: bit 0 set (default) = use the row-shared kernels for more

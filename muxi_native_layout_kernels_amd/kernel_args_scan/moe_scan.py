@@ -7,8 +7,10 @@ Counterpart of the reference's kernel_args_scan/muxi_moe_args_scan.py:92-110, wh
     one token          ids 2, 3 (row groups per workgroup and waves splitting K in the gate/up GeMV kernel),
                        4 (waves of the down kernel), 5 (16-byte loads in flight per wave)
     2 .. 16 tokens     id 7 (row groups per wave = K slices of the decode down kernel)
-    above 16 tokens    id 8 (upper limit of the 16-token blocks that share one pass over an expert's weights)
-                       and the row-shared kernels on / off (`mlk_moe_set_tile_path`)
+    above 16 tokens    id 8 (upper limit of the 16-token blocks that share one pass over an expert's weights),
+                       the row-shared kernels on / off (`mlk_moe_set_tile_path`) and, with soft-FP8 weights, id 10
+                       (panel kernels: K slices of the down projection + 16 x two workgroups per CU; ignored
+                       where the panel kernels do not run)
 
 Every setting is gated on the output of the default setting (rtol = atol = 1e-2, which the parity tests pin
 against the oracle), timed as HIP-graph replays of the whole `fused_moe` call, and the fastest one is written
@@ -35,7 +37,7 @@ PRESETS = {
     "deepseek_tp8": dict(experts=256, topk=8, hidden=7168, inter=256, grouped=True),
     "qwen3_30b": dict(experts=128, topk=8, hidden=2048, inter=768, grouped=True),
 }
-DEFAULTS = {2: 1, 3: 8, 4: 16, 5: 0, 7: 0, 8: 0}
+DEFAULTS = {2: 1, 3: 8, 4: 16, 5: 0, 7: 0, 8: 0, 10: 0}
 
 
 def _time_graph(call, iters):
@@ -63,7 +65,7 @@ def _time_graph(call, iters):
     return best
 
 
-def settings_for(tokens, topk):
+def settings_for(tokens, topk, fp8=False):
     """The grid of (tunable id -> value, tile path) settings that can matter at this token count."""
     if tokens == 1:
         out = []
@@ -74,7 +76,10 @@ def settings_for(tokens, topk):
         return out
     if tokens <= 16:
         return [({7: r}, 1) for r in (1, 2, 4)]
-    return [({8: cap}, tile) for cap, tile in itertools.product((0, 1, 2, 3, 4, 6, 8), (1, 0)) if tile or cap <= 4]
+    out = [({8: cap}, tile) for cap, tile in itertools.product((0, 1, 2, 3, 4, 6, 8), (1, 0)) if tile or cap <= 4]
+    if fp8:
+        out += [({10: v}, 1) for v in (1, 2, 4, 8, 17, 18, 20, 24)]
+    return out
 
 
 def apply(lib, setting):
@@ -114,7 +119,7 @@ def scan(experts, topk, hidden, inter, grouped, fp8, tokens, iters, out):
         want = call().float()
         us_default = _time_graph(call, iters)
         best = (us_default, ({}, 1))
-        for setting in settings_for(t, topk):
+        for setting in settings_for(t, topk, fp8):
             apply(lib, setting)
             try:
                 got = call().float()
